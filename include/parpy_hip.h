@@ -1,0 +1,83 @@
+/*
+ * C ABI of the ParPy HIP runtime library (libparpy_hip.so) for MI355X (gfx950).
+ *
+ * First group: the seven runtime entry points of the reference's native
+ * runtime, python/parpy/native/parpy_cuda.h:15-25 (bound from ctypes in
+ * python/parpy/runtime.py:11-26), with identical names, argument meaning and
+ * return conventions so that the reference's Python driver binds them
+ * unchanged.
+ *
+ * Second group: what replaces the reference's "generate a host translation
+ * unit, run nvcc, dlopen the result" step (python/parpy/compile.py:29-54,
+ * 123-184): runtime compilation of the generated device source with hiprtc,
+ * code-object loading, and execution of the generated launch plan with
+ * hipModuleLaunchKernel.  parpy_hip_plan_run plays the role of the generated
+ * `extern "C" int32_t <fun>(...)` entry point (src/gpu/codegen.rs:540-547):
+ * same flattened pointer arguments, same 0 / non-zero status, message through
+ * parpy_get_error_message.
+ *
+ * All work is enqueued on the null stream and is not synchronised before
+ * returning (like the reference).  No torch or Python types appear here.
+ * Thread-safety: none promised beyond what HIP gives; the error message is a
+ * per-thread buffer owned by the library.
+ */
+#ifndef PARPY_HIP_H
+#define PARPY_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- reference runtime surface (python/parpy/native/parpy_cuda.h:15-25) ---- */
+void parpy_init(int64_t unused);                                   /* parpy_cuda.cpp:3-5   */
+int32_t parpy_sync(void);                                          /* parpy_cuda.cpp:7-9   */
+void* parpy_alloc_buffer(int64_t nbytes);                          /* parpy_cuda.cpp:11-17; NULL on failure */
+int32_t parpy_memcpy(void* dst, void* src, int64_t nbytes, int64_t kind); /* :19-31; kind 0 H2H, 1 H2D, 2 D2H, 3 D2D */
+int32_t parpy_memset(void* ptr, int64_t nbytes, int8_t value);     /* parpy_cuda.cpp:33-35 */
+int32_t parpy_free_buffer(void* ptr);                              /* parpy_cuda.cpp:37-39 */
+const char* parpy_get_error_message(void);                         /* parpy_cuda.h:22-25   */
+
+/* ---- runtime compilation and loading (replaces python/parpy/compile.py:29-54) ---- */
+
+/* Compile HIP C++ `source` with hiprtc.  `options` are compiler flags; the
+ * target architecture defaults to gfx950 when no --offload-arch is given.
+ * On success *code / *size receive the code object (free it with
+ * parpy_hip_free_code).  On failure the hiprtc log is the error message.
+ * Does not need a GPU. */
+int32_t parpy_hip_compile(const char* source, const char* const* options,
+                          int32_t noptions, void** code, size_t* size);
+void parpy_hip_free_code(void* code);
+
+/* Load / unload a code object on the current device (hipModuleLoadData). */
+int32_t parpy_hip_module_load(const void* code, size_t size, void** module);
+int32_t parpy_hip_module_unload(void* module);
+
+/* Launch one kernel of a loaded module on the null stream
+ * (hipModuleLaunchKernel); `args` are pointers to the argument values. */
+int32_t parpy_hip_launch(void* module, const char* kernel,
+                         const int64_t grid[3], const int64_t block[3],
+                         int64_t lds_bytes, void** args);
+
+/* ---- launch plans (replaces the generated host entry point) ---- */
+
+/* Build an executable plan from the text emitted by parpy_hipc_compile.
+ * Kernel functions are resolved once, here. */
+int32_t parpy_hip_plan_create(void* module, const char* plan_text, void** plan);
+
+/* Run the plan: `args` are the flattened pointer arguments in call order
+ * (dict fields sorted by key, python/parpy/compile.py:142-146); scalars were
+ * folded into the code at compile time.  Returns 0 or non-zero. */
+int32_t parpy_hip_plan_run(void* plan, void* const* args, int32_t nargs);
+
+/* Number of kernel launches the last run of this plan enqueued. */
+int64_t parpy_hip_plan_launch_count(void* plan);
+
+int32_t parpy_hip_plan_destroy(void* plan);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

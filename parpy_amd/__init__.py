@@ -1,0 +1,169 @@
+"""parpy_amd: ParPy's user surface on an MI355X-native HIP backend.
+
+`import parpy_amd as parpy` gives the reference's API unchanged
+(python/parpy/__init__.py:1-246): jit, label, gpu, par, threads, reduce,
+CompileOptions, CompileBackend (+ Hip), print_compiled, compile_string,
+clear_cache, sync, buffer, types, operators, backend.
+"""
+from . import options
+from . import backend
+from . import buffer
+from . import operators
+from . import types
+from . import compiler
+
+from .options import par, CompileBackend, CompileOptions, ElemSize, Target, LoopPar, DataType, ScalarSizes
+from .buffer import sync
+from .operators import gpu, label
+
+__version__ = "0.1.3"
+
+_ir_asts = {}
+_ext_decls = {}
+_ext_tops = {}
+_fun_cache = {}
+
+
+def _get_tops(backend):
+    ast_tops = {k.__name__: v for k, v in _ir_asts.items()}
+    if backend is not None:
+        ext_tops = _ext_decls.get(backend, {})
+    else:
+        ext_tops = _ext_tops
+    return {**ast_tops, **ext_tops}
+
+
+def _get_source_code(fn):
+    import inspect
+    import itertools
+    import textwrap
+    src, fst_line = inspect.getsourcelines(fn)
+    col_ofs = sum(1 for _ in itertools.takewhile(str.isspace, src[0]))
+    src = textwrap.dedent("".join(src))
+    return src, fst_line - 1, col_ofs
+
+
+def _convert_python_function_to_ir(fn, vars):
+    import ast as python_ast
+    import inspect
+    filepath = inspect.getfile(fn)
+    src, line_ofs, col_ofs = _get_source_code(fn)
+    tree = python_ast.parse(src)
+    # a decorated function is parsed with its decorator lines: they do not belong to the body
+    top_map = _get_tops(None)
+    info = (filepath, line_ofs, col_ofs)
+    return compiler.python_to_ir(tree, info, top_map, vars)
+
+
+def _check_kwarg(kwargs, key, expected_ty, fun_name):
+    if key not in kwargs or kwargs[key] is None:
+        raise RuntimeError(f"Missing required keyword argument {key} in call to {fun_name}")
+    if isinstance(kwargs[key], expected_ty):
+        v = kwargs[key]
+        del kwargs[key]
+        return v
+    raise RuntimeError(f"The keyword argument {key} should be of type {expected_ty}")
+
+
+def _check_kwargs(kwargs, fun_name):
+    opts = _check_kwarg(kwargs, "opts", CompileOptions, fun_name)
+    if len(kwargs) > 0:
+        raise RuntimeError(f"Received unsupported keyword arguments: {kwargs}")
+    return opts
+
+
+def _compile_function(ir_ast, args, opts):
+    from .compile import build_code_object, get_wrapper
+    from .key import _generate_fast_cache_key, _generate_function_key
+    name = compiler.get_function_name(ir_ast)
+    fast_cache_key = _generate_fast_cache_key(ir_ast, args, opts)
+    if fast_cache_key in _fun_cache:
+        return _fun_cache[fast_cache_key]
+    top_map = _get_tops(opts.backend)
+    res = compiler.compile_ir(ir_ast, args, opts, top_map)
+    cache_key = _generate_function_key(res.device_src, opts)
+    build_code_object(cache_key, res.device_src, opts)
+    wrap_fn = get_wrapper(name, cache_key, res.plan, opts)
+    _fun_cache[fast_cache_key] = wrap_fn
+    return wrap_fn
+
+
+def threads(n):
+    """A LoopPar describing a parallel operation over `n` threads."""
+    return LoopPar().threads(n)
+
+
+def reduce():
+    """A LoopPar describing a parallelizable reduction."""
+    return LoopPar().reduce()
+
+
+def clear_cache():
+    """Clear the cached code objects and the in-memory function cache."""
+    from .compile import clear_cache as _clear
+    global _fun_cache
+    _clear()
+    _fun_cache = {}
+
+
+def compile_string(fun_name, code, opts=None, grid=(1, 1, 1), block=(64, 1, 1)):
+    """Compile HIP device code given as a string and return a launcher for kernel `fun_name`.
+
+    The reference compiles a host translation unit and calls its `extern "C"`
+    entry (python/parpy/__init__.py:161-178).  With runtime compilation there is
+    no host code, so the string holds `extern "C" __global__` kernels and the
+    launch dimensions are given here.
+    """
+    from .compile import build_code_object, get_string_wrapper
+    from .key import _generate_function_key
+    from .validate import check_arguments
+    import functools
+    opts = backend._resolve_backend(opts or CompileOptions(), True)
+    cache_key = "string_" + _generate_function_key(code, opts)
+    build_code_object(cache_key, code, opts)
+    fn = get_string_wrapper(fun_name, cache_key, grid, block, opts)
+
+    @functools.wraps(fn)
+    def inner(*args):
+        args = check_arguments(args, opts, True)
+        fn(*args)
+    return inner
+
+
+def print_compiled(fun, args, opts=None):
+    """Generated code (device source and host launch sequence) of `fun` for `args`; needs no GPU."""
+    from .validate import check_arguments
+    import inspect
+    opts = backend._resolve_backend(opts or CompileOptions(), False)
+    if fun in _ir_asts:
+        ir_ast = _ir_asts[fun]
+    else:
+        globs = inspect.currentframe().f_back.f_globals
+        locs = inspect.currentframe().f_back.f_locals
+        ir_ast = _convert_python_function_to_ir(fun, (globs, locs))
+    args = check_arguments(args, opts, False)
+    top_map = _get_tops(opts.backend)
+    return compiler.compile_ir(ir_ast, args, opts, top_map).listing
+
+
+def external(ext_name, backend, target, header=None, parallelize=LoopPar()):
+    """Declare an externally defined device function (not available in the HIP backend yet)."""
+    raise RuntimeError("External functions are not supported by the HIP backend yet")
+
+
+def jit(fun):
+    """Prepare `fun` for JIT compilation: parse once now, specialise on the arguments of each call."""
+    from .validate import check_arguments
+    import functools
+    import inspect
+    globs = inspect.currentframe().f_back.f_globals
+    locs = inspect.currentframe().f_back.f_locals
+    ir_ast = _convert_python_function_to_ir(fun, (globs, locs))
+
+    @functools.wraps(fun)
+    def inner(*args, **kwargs):
+        opts = backend._resolve_backend(_check_kwargs(kwargs, fun.__name__), True)
+        args = check_arguments(args, opts, True)
+        _compile_function(ir_ast, args, opts)(*args)
+    _ir_asts[inner] = ir_ast
+    return inner

@@ -1,0 +1,162 @@
+"""Build, cache, load and wrap compiled functions.
+
+Counterpart of python/parpy/compile.py of the reference.  What changes: the
+generated code is device-only HIP C++ compiled in-process by hiprtc (through
+the runtime library) instead of a host+device translation unit compiled by an
+nvcc subprocess, and the object that is loaded is a code object plus a launch
+plan instead of a shared library.  What stays: the on-disk cache keyed by the
+sha256 of the generated code and flags (python/parpy/compile.py:4-12,108-115),
+the error text of a failed build (:17-27), dict arguments expanded sorted by
+key (:142-146) and a non-zero status turned into RuntimeError with the runtime's
+message (:172-182).
+"""
+import ctypes
+import os
+from pathlib import Path
+
+cache_path = Path(os.environ.get("PARPY_CACHE_DIR", f"{os.path.expanduser('~')}/.cache/parpy_amd"))
+cache_path.mkdir(parents=True, exist_ok=True)
+
+# code generation flags for every generated kernel: no packed fp32 instructions
+HIPRTC_FLAGS = ["-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+_modules = {}   # key -> (module handle, code bytes) kept alive for the process lifetime
+
+
+def _get_code_path(key):
+    return cache_path / f"{key}.hsaco"
+
+
+def _is_cached(key):
+    return os.path.isfile(_get_code_path(key))
+
+
+def clear_cache():
+    """Remove every cached code object."""
+    import shutil
+    shutil.rmtree(f"{cache_path}", ignore_errors=True)
+    cache_path.mkdir(parents=True, exist_ok=True)
+    _modules.clear()
+
+
+def hiprtc_compile(source, opts, lib=None):
+    """Compile device source to a gfx950 code object (bytes).  Needs no GPU."""
+    from .runtime import load_hip_runtime_lib
+    lib = lib or load_hip_runtime_lib()
+    flags = list(HIPRTC_FLAGS) + [f"-I{inc}" for inc in opts.includes] + list(opts.extra_flags)
+    cflags = (ctypes.c_char_p * len(flags))(*[f.encode() for f in flags])
+    code = ctypes.c_void_p()
+    size = ctypes.c_size_t()
+    rc = lib.parpy_hip_compile(source.encode("utf-8"), cflags, len(flags), ctypes.byref(code), ctypes.byref(size))
+    if rc != 0:
+        msg = lib.parpy_get_error_message().decode("utf-8", "replace")
+        msg = f"Compilation of generated HIP code failed with exit code {rc}:\n{msg}"
+        if opts.write_output:
+            import uuid
+            temp_file = f"{uuid.uuid4().hex}.hip"
+            with open(temp_file, "w+") as f:
+                f.write(source)
+            msg += f"\nWrote generated code to file {temp_file}."
+        raise RuntimeError(msg)
+    data = ctypes.string_at(code.value, size.value)
+    lib.parpy_hip_free_code(code)
+    return data
+
+
+def build_code_object(key, source, opts):
+    """Compile `source` unless a code object for `key` is already cached on disk."""
+    from .options import CompileBackend
+    if opts.backend != CompileBackend.Hip:
+        raise RuntimeError(f"Cannot build for unsupported backend {opts.backend}")
+    path = _get_code_path(key)
+    if not _is_cached(key):
+        data = hiprtc_compile(source, opts)
+        tmp = path.with_suffix(f".tmp{os.getpid()}")
+        with open(tmp, "wb") as f:
+            f.write(data)
+        os.replace(tmp, path)
+    if opts.write_output:
+        with open(cache_path / f"{key}.hip", "w") as f:
+            f.write(source)
+    return path
+
+
+def _load_module(key, lib):
+    if key not in _modules:
+        with open(_get_code_path(key), "rb") as f:
+            data = f.read()
+        buf = ctypes.create_string_buffer(data, len(data))
+        module = ctypes.c_void_p()
+        rc = lib.parpy_hip_module_load(buf, len(data), ctypes.byref(module))
+        if rc != 0:
+            raise RuntimeError(lib.parpy_get_error_message().decode("ascii", "replace"))
+        _modules[key] = (module, buf)
+    return _modules[key][0]
+
+
+def _expand_arg(arg):
+    if isinstance(arg, dict):
+        return [v for (_, v) in sorted(arg.items())]
+    return [arg]
+
+
+def get_wrapper(name, key, plan_text, opts):
+    """Callable that runs the launch plan of a compiled function on its (validated) arguments."""
+    from .buffer import Buffer
+    from .runtime import _compile_runtime_lib
+    lib = _compile_runtime_lib(opts.backend)
+    module = _load_module(key, lib)
+    plan = ctypes.c_void_p()
+    rc = lib.parpy_hip_plan_create(module, plan_text.encode("utf-8"), ctypes.byref(plan))
+    if rc != 0:
+        raise RuntimeError(lib.parpy_get_error_message().decode("ascii", "replace"))
+
+    def wrapper(*args):
+        flat = [x for a in args for x in _expand_arg(a)]
+        # scalars and 0-d buffers were folded into the code; what is passed are array pointers
+        ptrs = [a._get_ptr() for a in flat if isinstance(a, Buffer) and len(a.shape) > 0]
+        arr = (ctypes.c_void_p * max(1, len(ptrs)))(*ptrs)
+        status = lib.parpy_hip_plan_run(plan, arr, len(ptrs))
+        if status != 0:
+            msg = lib.parpy_get_error_message()
+            raise RuntimeError(f"{msg.decode('ascii', 'replace')}")
+    wrapper.__name__ = name
+    wrapper.plan = plan
+    wrapper.launch_count = lambda: lib.parpy_hip_plan_launch_count(plan)
+    return wrapper
+
+
+def get_string_wrapper(kernel_name, key, grid, block, opts):
+    """Wrapper for parpy.compile_string: one hand-written kernel launched with a fixed grid."""
+    from .buffer import Buffer
+    from .options import ScalarSizes
+    from .runtime import _compile_runtime_lib
+    lib = _compile_runtime_lib(opts.backend)
+    module = _load_module(key, lib)
+    sizes = ScalarSizes(opts)
+    g = (ctypes.c_int64 * 3)(*grid)
+    b = (ctypes.c_int64 * 3)(*block)
+
+    def wrapper(*args):
+        flat = [x for a in args for x in _expand_arg(a)]
+        storage = []
+        for a in flat:
+            if isinstance(a, bool):
+                storage.append(ctypes.c_bool(a))
+            elif isinstance(a, int):
+                storage.append(sizes.int.to_ctype()(a))
+            elif isinstance(a, float):
+                storage.append(sizes.float.to_ctype()(a))
+            elif isinstance(a, Buffer):
+                if len(a.shape) == 0:
+                    storage.append(a.dtype.to_ctype()(a.numpy().item()))
+                else:
+                    storage.append(ctypes.c_void_p(a._get_ptr()))
+            else:
+                raise RuntimeError(f"Argument {a} has unsupported type {type(a)}")
+        ptrs = (ctypes.c_void_p * max(1, len(storage)))(*[ctypes.cast(ctypes.pointer(s), ctypes.c_void_p) for s in storage])
+        status = lib.parpy_hip_launch(module, kernel_name.encode(), ctypes.byref(g), ctypes.byref(b), 0, ptrs)
+        if status != 0:
+            raise RuntimeError(lib.parpy_get_error_message().decode("ascii", "replace"))
+    wrapper.__name__ = kernel_name
+    return wrapper

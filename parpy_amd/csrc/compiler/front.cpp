@@ -1,0 +1,443 @@
+// Decoration-time front end: S-expression -> untyped AST, symbol binding,
+// label association and inlining of statement calls.
+//
+// Counterpart of the reference's src/py/mod.rs:34-43 (parse_untyped_ast),
+// src/py/symbolize.rs, src/py/labels.rs:16-98 and src/py/inline_calls.rs:13-111.
+#include "passes.hpp"
+
+namespace parpy {
+
+namespace {
+
+Info parse_info(const SXP& a) {
+  Info i;
+  if (a->is_list || a->atom.empty() || a->atom[0] != '@') return i;
+  sscanf(a->atom.c_str(), "@%d:%d:%d:%d", &i.l0, &i.c0, &i.l1, &i.c1);
+  return i;
+}
+
+struct Reader {
+  std::shared_ptr<Expr> node(Expr::Kind k, const Info& i) {
+    auto e = std::make_shared<Expr>();
+    e->k = k;
+    e->ty = Type();
+    e->i = i;
+    return e;
+  }
+
+  UnOp unop(const std::string& s, const Info& i) {
+    if (s == "sub") return UnOp::Sub;
+    if (s == "not") return UnOp::Not;
+    if (s == "bitneg") return UnOp::BitNeg;
+    fail_rt(i, "Unsupported unary expression " + s);
+  }
+
+  BinOp binop(const std::string& s, const Info& i) {
+    static const std::map<std::string, BinOp> m = {
+        {"add", BinOp::Add}, {"sub", BinOp::Sub}, {"mul", BinOp::Mul}, {"div", BinOp::Div},
+        {"floordiv", BinOp::FloorDiv}, {"rem", BinOp::Rem}, {"pow", BinOp::Pow}, {"and", BinOp::And},
+        {"or", BinOp::Or}, {"bitand", BinOp::BitAnd}, {"bitor", BinOp::BitOr}, {"bitxor", BinOp::BitXor},
+        {"shl", BinOp::BitShl}, {"shr", BinOp::BitShr}, {"eq", BinOp::Eq}, {"neq", BinOp::Neq},
+        {"leq", BinOp::Leq}, {"geq", BinOp::Geq}, {"lt", BinOp::Lt}, {"gt", BinOp::Gt}};
+    auto it = m.find(s);
+    if (it == m.end()) fail_rt(i, "Unsupported binary operation: " + s);
+    return it->second;
+  }
+
+  E expr(const SXP& x) {
+    if (!x->is_list || x->size() < 2) throw std::runtime_error("malformed expression node");
+    const std::string& h = x->head();
+    Info i = parse_info(x->at(1));
+    if (h == "var") {
+      auto e = node(Expr::Var, i);
+      e->name = Name{x->at(2)->atom, 0};
+      return e;
+    }
+    if (h == "int") { auto e = node(Expr::Int, i); e->iv = x->at(2)->as_int(); return e; }
+    if (h == "float") { auto e = node(Expr::Float, i); e->fv = x->at(2)->as_double(); return e; }
+    if (h == "bool") { auto e = node(Expr::Bool, i); e->bv = x->at(2)->atom == "true"; return e; }
+    if (h == "str") { auto e = node(Expr::Str, i); e->sval = x->at(2)->atom; return e; }
+    if (h == "unop") {
+      auto e = node(Expr::UnOpE, i);
+      e->uop = unop(x->at(2)->atom, i);
+      e->args = {expr(x->at(3))};
+      return e;
+    }
+    if (h == "binop") {
+      auto e = node(Expr::BinOpE, i);
+      e->bop = binop(x->at(2)->atom, i);
+      e->args = {expr(x->at(3)), expr(x->at(4))};
+      return e;
+    }
+    if (h == "ifexp") {
+      auto e = node(Expr::IfExpr, i);
+      e->args = {expr(x->at(2)), expr(x->at(3)), expr(x->at(4))};
+      return e;
+    }
+    if (h == "sub") {
+      auto e = node(Expr::Subscript, i);
+      e->args = {expr(x->at(2)), expr(x->at(3))};
+      return e;
+    }
+    if (h == "slice") {
+      auto e = node(Expr::Slice, i);
+      e->args = {x->at(2)->is_sym("none") ? E() : expr(x->at(2)), x->at(3)->is_sym("none") ? E() : expr(x->at(3))};
+      return e;
+    }
+    if (h == "tuple") {
+      auto e = node(Expr::Tuple, i);
+      for (size_t k = 2; k < x->size(); ++k) e->args.push_back(expr(x->at(k)));
+      return e;
+    }
+    if (h == "call") {
+      auto e = node(Expr::Call, i);
+      e->sval = x->at(2)->atom;
+      for (size_t k = 3; k < x->size(); ++k) e->args.push_back(expr(x->at(k)));
+      return e;
+    }
+    if (h == "builtin") {
+      auto e = node(Expr::BuiltinE, i);
+      const std::string& n = x->at(2)->atom;
+      static const std::map<std::string, Builtin> m = {
+          {"exp", Builtin::Exp}, {"inf", Builtin::Inf}, {"log", Builtin::Log}, {"min", Builtin::Min},
+          {"max", Builtin::Max}, {"abs", Builtin::Abs}, {"cos", Builtin::Cos}, {"sin", Builtin::Sin},
+          {"sqrt", Builtin::Sqrt}, {"tanh", Builtin::Tanh}, {"atan2", Builtin::Atan2}, {"sum", Builtin::Sum},
+          {"prod", Builtin::Prod}, {"label", Builtin::Label}, {"gpu", Builtin::Gpu}};
+      if (n.rfind("convert_", 0) == 0) {
+        e->fn = Builtin::Convert;
+        ElemSize sz;
+        if (!parse_elem_tag(n.substr(8), &sz)) fail_rt(i, "Unknown conversion " + n);
+        e->ty = Type::scalar(sz);  // target type is carried in ty until type checking
+      } else {
+        auto it = m.find(n);
+        if (it == m.end()) fail_rt(i, "Unknown built-in operator " + n);
+        e->fn = it->second;
+      }
+      if (!x->at(3)->is_sym("none")) { e->has_axis = true; e->iv = x->at(3)->as_int(); }
+      for (size_t k = 4; k < x->size(); ++k) e->args.push_back(expr(x->at(k)));
+      return e;
+    }
+    throw std::runtime_error("unknown expression node '" + h + "'");
+  }
+
+  Stmts stmts(const SXP& lst, size_t from = 1) {
+    Stmts r;
+    for (size_t k = from; k < lst->size(); ++k) r.push_back(stmt(lst->at(k)));
+    return r;
+  }
+
+  S stmt(const SXP& x) {
+    const std::string& h = x->head();
+    Info i = parse_info(x->at(1));
+    auto s = std::make_shared<Stmt>();
+    s->i = i;
+    if (h == "for") {
+      s->k = Stmt::For;
+      s->id = Name{x->at(2)->atom, 0};
+      s->lo = expr(x->at(3));
+      s->hi = expr(x->at(4));
+      s->step = x->at(5)->as_int();
+      s->body = stmts(x->at(6));
+      s->par = LoopPar();
+    } else if (h == "while") {
+      s->k = Stmt::While;
+      s->expr = expr(x->at(2));
+      s->body = stmts(x->at(3));
+    } else if (h == "if") {
+      s->k = Stmt::If;
+      s->expr = expr(x->at(2));
+      s->body = stmts(x->at(3));
+      s->els = stmts(x->at(4));
+    } else if (h == "assign") {
+      s->k = Stmt::Assign;
+      s->dst = expr(x->at(2));
+      s->expr = expr(x->at(3));
+    } else if (h == "withgpu") {
+      s->k = Stmt::WithGpu;
+      s->body = stmts(x->at(2));
+    } else if (h == "callstmt") {
+      s->k = Stmt::CallStmt;
+      s->fname = x->at(2)->atom;
+      for (size_t k = 3; k < x->size(); ++k) s->args.push_back(expr(x->at(k)));
+    } else if (h == "label") {
+      s->k = Stmt::Label;
+      s->fname = x->at(2)->atom;
+    } else if (h == "return") {
+      s->k = Stmt::Return;
+      s->expr = expr(x->at(2));
+    } else {
+      throw std::runtime_error("unknown statement node '" + h + "'");
+    }
+    return s;
+  }
+
+  Type annotation(const SXP& x, const Info& i) {
+    if (x->is_sym("none")) return Type();
+    ElemSize sz;
+    if (!x->is_list || x->size() != 2 || !parse_elem_tag(x->at(1)->atom, &sz))
+      fail_rt(i, "Unsupported parameter type annotation");
+    if (x->head() == "scalar") return Type::scalar(sz);
+    if (x->head() == "pointer") return Type::pointer(sz);
+    fail_rt(i, "Unsupported parameter type annotation");
+  }
+
+  FunDef fun(const SXP& x) {
+    if (x->head() != "fun") throw std::runtime_error("expected (fun ...)");
+    FunDef f;
+    f.id = Name{x->at(1)->atom, 0};
+    f.i = parse_info(x->at(2));
+    f.res_ty = annotation(x->at(3), f.i);
+    const SXP& ps = x->at(4);
+    for (size_t k = 1; k < ps->size(); ++k) {
+      const SXP& p = ps->at(k);
+      Param q;
+      q.id = Name{p->at(1)->atom, 0};
+      q.i = parse_info(p->at(3));
+      q.ty = annotation(p->at(2), q.i);
+      f.params.push_back(q);
+    }
+    f.body = stmts(x->at(5));
+    return f;
+  }
+};
+
+// ---------------------------------------------------------------- symbolize
+// The first assignment to a name that is not bound in an enclosing scope
+// becomes a definition (src/py/symbolize.rs:104-122).  Scopes follow the block
+// structure because the emitted code is C++.
+struct Symbolizer {
+  NameGen& gen;
+  std::vector<std::map<std::string, Name>> scopes;
+
+  explicit Symbolizer(NameGen& g) : gen(g) {}
+
+  const Name* lookup(const std::string& s) const {
+    for (auto it = scopes.rbegin(); it != scopes.rend(); ++it) {
+      auto f = it->find(s);
+      if (f != it->end()) return &f->second;
+    }
+    return nullptr;
+  }
+
+  E expr(const E& e) {
+    if (!e) return e;
+    if (e->k == Expr::Var) {
+      if (e->name.id != 0) return e;
+      const Name* n = lookup(e->name.s);
+      if (!n) fail_name(e->i, "Found reference to unknown variable " + e->name.s);
+      auto r = std::make_shared<Expr>(*e);
+      r->name = *n;
+      return r;
+    }
+    return map_children(e, [&](const E& c) { return expr(c); });
+  }
+
+  Stmts block(const Stmts& ss) {
+    scopes.emplace_back();
+    Stmts r;
+    for (auto& s : ss) r.push_back(stmt(s));
+    scopes.pop_back();
+    return r;
+  }
+
+  S stmt(const S& s) {
+    auto r = std::make_shared<Stmt>(*s);
+    switch (s->k) {
+      case Stmt::Assign: {
+        r->expr = expr(s->expr);
+        if (s->dst->k == Expr::Var && !lookup(s->dst->name.s)) {
+          r->k = Stmt::Def;
+          r->id = gen.fresh(s->dst->name.s);
+          r->ty = Type();
+          r->dst = nullptr;
+          scopes.back()[r->id.s] = r->id;
+        } else {
+          r->dst = expr(s->dst);
+        }
+        break;
+      }
+      case Stmt::For: {
+        r->lo = expr(s->lo);
+        r->hi = expr(s->hi);
+        scopes.emplace_back();
+        r->id = gen.fresh(s->id.s);
+        scopes.back()[r->id.s] = r->id;
+        r->body = block(s->body);
+        scopes.pop_back();
+        break;
+      }
+      case Stmt::While:
+        r->expr = expr(s->expr);
+        r->body = block(s->body);
+        break;
+      case Stmt::If:
+        r->expr = expr(s->expr);
+        r->body = block(s->body);
+        r->els = block(s->els);
+        break;
+      case Stmt::WithGpu: {
+        // a GPU context is transparent for scoping: what it defines stays visible after it
+        Stmts b;
+        for (auto& c : s->body) b.push_back(stmt(c));
+        r->body = b;
+        break;
+      }
+      case Stmt::CallStmt:
+        for (auto& a : r->args) a = expr(a);
+        break;
+      case Stmt::Return:
+        r->expr = expr(s->expr);
+        break;
+      default:
+        break;
+    }
+    return r;
+  }
+};
+
+// ---------------------------------------------------------------- labels
+S add_labels(const S& s, std::vector<std::string>& l) {
+  if (s->k != Stmt::Def && s->k != Stmt::Assign && s->k != Stmt::For)
+    fail_rt(s->i, "Cannot associate label with non-parallelizable statement");
+  auto r = std::make_shared<Stmt>(*s);
+  for (auto& x : l) r->labels.push_back(x);
+  l.clear();
+  return r;
+}
+
+Stmts associate_labels(const Stmts& ss) {
+  Stmts out;
+  std::vector<std::string> labels;
+  for (auto& s0 : ss) {
+    if (s0->k == Stmt::Label) {
+      labels.push_back(s0->fname);
+      continue;
+    }
+    S s = labels.empty() ? s0 : add_labels(s0, labels);
+    if (!s->body.empty() || !s->els.empty()) {
+      auto r = std::make_shared<Stmt>(*s);
+      r->body = associate_labels(s->body);
+      r->els = associate_labels(s->els);
+      s = r;
+    }
+    out.push_back(s);
+  }
+  if (!labels.empty())
+    fail_rt(out.empty() ? Info() : out.back()->i, "Found labels not associated with any statement");
+  return out;
+}
+
+// ---------------------------------------------------------------- inlining of statement calls
+struct Inliner {
+  NameGen& gen;
+  const std::map<std::string, const ParsedFun*>& tops;
+
+  // substitute parameters by argument expressions and give every callee-local
+  // name a fresh identity in the caller
+  struct Sub {
+    std::map<Name, E> params;
+    std::map<Name, Name> locals;
+  };
+
+  E sub_expr(const E& e, Sub& sub) {
+    if (!e) return e;
+    if (e->k == Expr::Var) {
+      auto p = sub.params.find(e->name);
+      if (p != sub.params.end()) {
+        auto r = std::make_shared<Expr>(*p->second);
+        r->i = e->i;
+        return r;
+      }
+      auto l = sub.locals.find(e->name);
+      if (l != sub.locals.end()) {
+        auto r = std::make_shared<Expr>(*e);
+        r->name = l->second;
+        return r;
+      }
+      return e;
+    }
+    return map_children(e, [&](const E& c) { return sub_expr(c, sub); });
+  }
+
+  Stmts sub_stmts(const Stmts& ss, Sub& sub) {
+    Stmts out;
+    for (auto& s : ss) {
+      auto r = std::make_shared<Stmt>(*s);
+      if (s->k == Stmt::Def || s->k == Stmt::For) {
+        Name n = gen.fresh(s->id.s);
+        sub.locals[s->id] = n;
+        r->id = n;
+      }
+      if (s->k == Stmt::Return) fail_rt(s->i, "Cannot inline a call to a function containing a return statement");
+      if (r->dst) {
+        if (r->dst->k == Expr::Var && sub.params.count(r->dst->name) && sub.params[r->dst->name]->k != Expr::Var)
+          fail_rt(s->i, "Cannot assign to a parameter bound to a non-variable argument in an inlined call");
+        r->dst = sub_expr(r->dst, sub);
+      }
+      if (r->expr) r->expr = sub_expr(r->expr, sub);
+      if (r->lo) r->lo = sub_expr(r->lo, sub);
+      if (r->hi) r->hi = sub_expr(r->hi, sub);
+      for (auto& a : r->args) a = sub_expr(a, sub);
+      r->body = sub_stmts(s->body, sub);
+      r->els = sub_stmts(s->els, sub);
+      out.push_back(r);
+    }
+    return out;
+  }
+
+  Stmts run(const Stmts& ss) {
+    Stmts out;
+    for (auto& s : ss) {
+      if (s->k == Stmt::CallStmt) {
+        auto it = tops.find(s->fname);
+        if (it == tops.end()) fail_rt(s->i, "Reference to unknown function " + s->fname + ".");
+        const FunDef& f = it->second->fun;
+        if (f.params.size() != s->args.size())
+          fail_rt(f.i, "Function " + f.id.s + " expected " + std::to_string(f.params.size()) +
+                           " arguments, but received " + std::to_string(s->args.size()) + ".");
+        Sub sub;
+        for (size_t k = 0; k < f.params.size(); ++k) sub.params[f.params[k].id] = s->args[k];
+        Stmts body = sub_stmts(f.body, sub);
+        for (auto& b : body) out.push_back(b);
+        continue;
+      }
+      if (s->body.empty() && s->els.empty()) {
+        out.push_back(s);
+        continue;
+      }
+      auto r = std::make_shared<Stmt>(*s);
+      r->body = run(s->body);
+      r->els = run(s->els);
+      out.push_back(r);
+    }
+    return out;
+  }
+};
+
+}  // namespace
+
+std::unique_ptr<ParsedFun> parse_function(const std::string& sexpr,
+                                          const std::map<std::string, const ParsedFun*>& tops) {
+  SXP x = parse_sexpr(sexpr);
+  auto pf = std::make_unique<ParsedFun>();
+  Reader rd;
+  pf->fun = rd.fun(x);
+
+  // symbolize: parameters first, then the body
+  Symbolizer sym(pf->gen);
+  sym.scopes.emplace_back();
+  for (auto& p : pf->fun.params) {
+    p.id = pf->gen.fresh(p.id.s);
+    sym.scopes.back()[p.id.s] = p.id;
+  }
+  Stmts body;
+  for (auto& s : pf->fun.body) body.push_back(sym.stmt(s));
+  pf->fun.body = associate_labels(body);
+
+  Inliner inl{pf->gen, tops};
+  pf->fun.body = inl.run(pf->fun.body);
+  pf->source_text = print_fun(pf->fun);
+  return pf;
+}
+
+}  // namespace parpy

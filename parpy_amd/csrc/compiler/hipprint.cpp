@@ -1,0 +1,728 @@
+// HIP C++ (gfx950) pretty-printer: device source for hiprtc, the host launch
+// plan for the runtime, and a combined human-readable listing.
+//
+// Takes the place of the reference's src/cuda/pprint.rs:40-570 and
+// src/cuda/codegen.rs:120-358.  There is no generated host translation unit:
+// host loops, temporaries and launches are emitted as a launch plan that the
+// runtime library interprets (hipModuleLaunchKernel), so nothing but device
+// code goes through a compiler at call time.
+#include <cinttypes>
+#include <sstream>
+
+#include "passes.hpp"
+
+namespace parpy {
+
+namespace {
+
+std::string fmt_f32(double v) {
+  if (std::isinf(v)) return v > 0 ? "__builtin_huge_valf()" : "(-__builtin_huge_valf())";
+  if (std::isnan(v)) return "__builtin_nanf(\"\")";
+  char buf[64];
+  snprintf(buf, sizeof buf, "%.9g", v);
+  std::string s = buf;
+  if (s.find('.') == std::string::npos && s.find('e') == std::string::npos) s += ".0";
+  return s + "f";
+}
+
+std::string fmt_f64(double v) {
+  if (std::isinf(v)) return v > 0 ? "__builtin_huge_val()" : "(-__builtin_huge_val())";
+  if (std::isnan(v)) return "__builtin_nan(\"\")";
+  char buf[64];
+  snprintf(buf, sizeof buf, "%.17g", v);
+  std::string s = buf;
+  if (s.find('.') == std::string::npos && s.find('e') == std::string::npos) s += ".0";
+  return s;
+}
+
+const char* red_suffix(BinOp op) {
+  switch (op) {
+    case BinOp::Add: return "add";
+    case BinOp::Mul: return "mul";
+    case BinOp::Max: return "max";
+    case BinOp::Min: return "min";
+    case BinOp::BitAnd: case BinOp::And: return "and";
+    case BinOp::BitOr: case BinOp::Or: return "or";
+    case BinOp::BitXor: return "xor";
+    default: return "add";
+  }
+}
+
+// Device helpers shared by all generated kernels.  Cross-lane reductions use
+// DPP row operations inside each row of 16 lanes, row broadcasts across the
+// four rows of a 64-lane wavefront, and a readlane broadcast so that every
+// lane ends up holding the result.
+const char* PREAMBLE = R"(#if defined(__HIPCC_RTC__)
+typedef signed char int8_t;
+typedef short int16_t;
+typedef int int32_t;
+typedef long long int64_t;
+typedef unsigned char uint8_t;
+typedef unsigned short uint16_t;
+typedef unsigned int uint32_t;
+typedef unsigned long long uint64_t;
+#else
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#endif
+
+template <int CTRL, class T> __device__ __forceinline__ T parpy_dpp(T v) {
+  if constexpr (sizeof(T) == 8) {
+    unsigned long long x = __builtin_bit_cast(unsigned long long, v);
+    int lo = (int)(unsigned)x, hi = (int)(unsigned)(x >> 32);
+    lo = __builtin_amdgcn_update_dpp(lo, lo, CTRL, 0xF, 0xF, false);
+    hi = __builtin_amdgcn_update_dpp(hi, hi, CTRL, 0xF, 0xF, false);
+    x = ((unsigned long long)(unsigned)hi << 32) | (unsigned)lo;
+    return __builtin_bit_cast(T, x);
+  } else if constexpr (sizeof(T) == 4) {
+    int x = __builtin_bit_cast(int, v);
+    x = __builtin_amdgcn_update_dpp(x, x, CTRL, 0xF, 0xF, false);
+    return __builtin_bit_cast(T, x);
+  } else {
+    int x = (int)v;
+    x = __builtin_amdgcn_update_dpp(x, x, CTRL, 0xF, 0xF, false);
+    return (T)x;
+  }
+}
+template <class T> __device__ __forceinline__ T parpy_readlane(T v, int lane) {
+  if constexpr (sizeof(T) == 8) {
+    unsigned long long x = __builtin_bit_cast(unsigned long long, v);
+    unsigned lo = (unsigned)__builtin_amdgcn_readlane((int)(unsigned)x, lane);
+    unsigned hi = (unsigned)__builtin_amdgcn_readlane((int)(unsigned)(x >> 32), lane);
+    x = ((unsigned long long)hi << 32) | lo;
+    return __builtin_bit_cast(T, x);
+  } else if constexpr (sizeof(T) == 4) {
+    return __builtin_bit_cast(T, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+  } else {
+    return (T)__builtin_amdgcn_readlane((int)v, lane);
+  }
+}
+struct parpy_op_add { template <class T> __device__ __forceinline__ T operator()(T a, T b) const { return a + b; } };
+struct parpy_op_mul { template <class T> __device__ __forceinline__ T operator()(T a, T b) const { return a * b; } };
+struct parpy_op_and { template <class T> __device__ __forceinline__ T operator()(T a, T b) const { return a & b; } };
+struct parpy_op_or { template <class T> __device__ __forceinline__ T operator()(T a, T b) const { return a | b; } };
+struct parpy_op_xor { template <class T> __device__ __forceinline__ T operator()(T a, T b) const { return a ^ b; } };
+struct parpy_op_max {
+  __device__ __forceinline__ float operator()(float a, float b) const { return fmaxf(a, b); }
+  __device__ __forceinline__ double operator()(double a, double b) const { return fmax(a, b); }
+  template <class T> __device__ __forceinline__ T operator()(T a, T b) const { return a > b ? a : b; }
+};
+struct parpy_op_min {
+  __device__ __forceinline__ float operator()(float a, float b) const { return fminf(a, b); }
+  __device__ __forceinline__ double operator()(double a, double b) const { return fmin(a, b); }
+  template <class T> __device__ __forceinline__ T operator()(T a, T b) const { return a < b ? a : b; }
+};
+template <class T> __device__ __forceinline__ T parpy_max(T a, T b) { return parpy_op_max()(a, b); }
+template <class T> __device__ __forceinline__ T parpy_min(T a, T b) { return parpy_op_min()(a, b); }
+// reduce over each row of 16 lanes; afterwards every lane of a row holds the row's result
+template <class Op, class T> __device__ __forceinline__ T parpy_row_reduce(T v) {
+  Op op;
+  v = op(v, parpy_dpp<0xB1>(v));   // quad_perm [1,0,3,2]
+  v = op(v, parpy_dpp<0x4E>(v));   // quad_perm [2,3,0,1]
+  v = op(v, parpy_dpp<0x141>(v));  // row_half_mirror
+  v = op(v, parpy_dpp<0x140>(v));  // row_mirror
+  return v;
+}
+// reduce over the 64 lanes of a wavefront; every lane receives the result
+template <class Op, class T> __device__ __forceinline__ T parpy_wave_reduce(T v) {
+  Op op;
+  v = parpy_row_reduce<Op>(v);
+  v = op(v, parpy_dpp<0x142>(v));  // row_bcast:15 (lane 15 of each row into the next row)
+  v = op(v, parpy_dpp<0x143>(v));  // row_bcast:31 (lane 31 into rows 2 and 3)
+  return parpy_readlane(v, 63);
+}
+// block reduction: one LDS slot per wavefront, then every wavefront reduces the partials
+template <class Op, int NWAVES, class T>
+__device__ __forceinline__ T parpy_block_reduce(T v, T neutral, T* slots, bool sync_after) {
+  v = parpy_wave_reduce<Op>(v);
+  if constexpr (NWAVES > 1) {
+    const int lane = threadIdx.x & 63;
+    if (lane == 0) slots[threadIdx.x >> 6] = v;
+    __syncthreads();
+    v = lane < NWAVES ? slots[lane] : neutral;
+    v = parpy_row_reduce<Op>(v);
+    v = parpy_readlane(v, 0);
+    if (sync_after) __syncthreads();
+  }
+  return v;
+}
+)";
+
+struct PE {  // printed integer expression: text + whether it was computed in 32-bit arithmetic
+  std::string s;
+  bool narrow = false;
+};
+
+bool fits32(const Interval& r) { return r.known && r.lo >= INT32_MIN && r.hi <= INT32_MAX; }
+
+struct DevicePrinter {
+  const Options& opts;
+  const Kernel* kernel = nullptr;
+  RangeEnv ranges;
+  std::set<Name> narrow_vars;     // 64-bit integer variables declared as 32-bit because their range allows it
+  std::set<Name> reassigned;      // variables assigned after their definition (their range is not tracked)
+  std::ostringstream os;
+  int red_sites = 0;
+  std::vector<std::string> lds_decls;
+
+  explicit DevicePrinter(const Options& o) : opts(o) {}
+
+  std::string ind(int n) { return std::string(n, ' '); }
+
+  // ---------------------------------------------------------------- expressions
+  std::string ctype(const Type& t) {
+    if (t.k == Type::Pointer) return std::string(elem_ctype(t.sz)) + "*";
+    if (t.k == Type::Tensor && !t.shape.empty()) return std::string(elem_ctype(t.sz)) + "*";
+    if (t.k == Type::Tensor) return elem_ctype(t.sz);
+    return "void";
+  }
+
+  std::string idx_name(Expr::Kind k, int dim) {
+    return std::string(k == Expr::ThreadIdx ? "threadIdx." : "blockIdx.") + "xyz"[dim];
+  }
+
+  bool is_i64(const E& e) { return e->ty.is_scalar() && (e->ty.sz == ElemSize::I64); }
+
+  // integer expressions whose semantic type is int64 are computed in 32 bits
+  // when interval analysis proves that neither the result nor any intermediate
+  // value leaves the int32 range
+  PE pint(const E& e) {
+    PE r;
+    if (!opts.opt_narrow_index || !is_i64(e)) { r.s = pexpr_plain(e); return r; }
+    switch (e->k) {
+      case Expr::Int:
+        if (e->iv >= INT32_MIN && e->iv <= INT32_MAX) { r.s = std::to_string(e->iv); r.narrow = true; }
+        else r.s = "((int64_t)" + std::to_string(e->iv) + "LL)";
+        return r;
+      case Expr::Var:
+        r.s = e->name.str();
+        r.narrow = narrow_vars.count(e->name) > 0;
+        return r;
+      case Expr::ThreadIdx: case Expr::BlockIdx:
+        r.s = "(int)" + idx_name(e->k, (int)e->iv);
+        r.narrow = true;
+        return r;
+      case Expr::Convert: {
+        const E& a = e->args[0];
+        if (a->ty.is_scalar() && is_int(a->ty.sz) && elem_bytes(a->ty.sz) <= 4 && !(a->ty.sz == ElemSize::U32)) {
+          r.s = "(int)" + paren(pexpr(a));
+          r.narrow = true;
+          return r;
+        }
+        r.s = pexpr_plain(e);
+        return r;
+      }
+      case Expr::BinOpE: {
+        BinOp op = e->bop;
+        bool arith = op == BinOp::Add || op == BinOp::Sub || op == BinOp::Mul || op == BinOp::FloorDiv ||
+                     op == BinOp::Div || op == BinOp::Rem || op == BinOp::BitAnd || op == BinOp::BitOr ||
+                     op == BinOp::BitXor || op == BinOp::BitShl || op == BinOp::BitShr || op == BinOp::Max || op == BinOp::Min;
+        if (!arith) { r.s = pexpr_plain(e); return r; }
+        PE a = pint(e->args[0]), b = pint(e->args[1]);
+        bool ok = a.narrow && b.narrow && fits32(expr_range(e, ranges));
+        std::string as = a.s, bs = b.s;
+        if (!ok) {
+          if (a.narrow) as = "(int64_t)" + paren(as);
+          if (b.narrow) bs = "(int64_t)" + paren(bs);
+        }
+        r.narrow = ok;
+        if (op == BinOp::Max || op == BinOp::Min)
+          r.s = std::string(op == BinOp::Max ? "parpy_max" : "parpy_min") + (ok ? "<int>(" : "<int64_t>(") + as + ", " + bs + ")";
+        else
+          r.s = "(" + as + " " + cop(op) + " " + bs + ")";
+        return r;
+      }
+      default:
+        r.s = pexpr_plain(e);
+        return r;
+    }
+  }
+
+  static std::string paren(const std::string& s) {
+    if (!s.empty() && s.front() == '(' && s.back() == ')') {
+      int depth = 0;
+      bool wraps = true;
+      for (size_t k = 0; k < s.size(); ++k) {
+        if (s[k] == '(') ++depth;
+        else if (s[k] == ')') { --depth; if (depth == 0 && k + 1 != s.size()) { wraps = false; break; } }
+      }
+      if (wraps) return s;
+    }
+    return "(" + s + ")";
+  }
+
+  static const char* cop(BinOp op) {
+    switch (op) {
+      case BinOp::FloorDiv: return "/";
+      case BinOp::Pow: return "**";
+      default: return binop_name(op);
+    }
+  }
+
+  std::string math_fn(const char* base, ElemSize sz, bool fast) {
+    // single precision uses the hardware approximations (v_exp_f32, v_log_f32, ...)
+    // like the reference's CUDA backend does (src/cuda/pprint.rs:70-92)
+    if (sz == ElemSize::F64) return base;
+    if (fast) return std::string("__") + base + "f";
+    return std::string(base) + "f";
+  }
+
+  std::string pexpr(const E& e) {
+    if (is_i64(e)) return pint(e).s;
+    return pexpr_plain(e);
+  }
+
+  std::string pexpr_plain(const E& e) {
+    switch (e->k) {
+      case Expr::Var: return e->name.str();
+      case Expr::Int: {
+        if (e->ty.is_scalar() && elem_bytes(e->ty.sz) == 8) {
+          if (e->ty.sz == ElemSize::U64) return "((uint64_t)" + std::to_string((uint64_t)e->iv) + "ULL)";
+          if (e->iv == INT64_MIN) return "((int64_t)(-9223372036854775807LL - 1))";
+          return "((int64_t)" + std::to_string(e->iv) + "LL)";
+        }
+        if (e->ty.is_scalar() && e->ty.sz != ElemSize::I32) return "((" + std::string(elem_ctype(e->ty.sz)) + ")" + std::to_string(e->iv) + ")";
+        return std::to_string(e->iv);
+      }
+      case Expr::Float:
+        if (e->ty.sz == ElemSize::F64) return fmt_f64(e->fv);
+        if (e->ty.sz == ElemSize::F16) return "((_Float16)" + fmt_f32(e->fv) + ")";
+        return fmt_f32(e->fv);
+      case Expr::Bool: return e->bv ? "true" : "false";
+      case Expr::UnOpE: {
+        std::string a = pexpr(e->args[0]);
+        ElemSize sz = e->ty.sz;
+        bool f16 = sz == ElemSize::F16;
+        auto call = [&](const std::string& fn) {
+          if (f16) return "((_Float16)" + fn + "((float)" + paren(a) + "))";
+          return fn + paren(a);
+        };
+        switch (e->uop) {
+          case UnOp::Sub: return "(-" + a + ")";
+          case UnOp::Not: return "(!" + a + ")";
+          case UnOp::BitNeg: return "(~" + a + ")";
+          case UnOp::Exp: return call(math_fn("exp", f16 ? ElemSize::F32 : sz, true));
+          case UnOp::Log: return call(math_fn("log", f16 ? ElemSize::F32 : sz, true));
+          case UnOp::Cos: return call(math_fn("cos", f16 ? ElemSize::F32 : sz, true));
+          case UnOp::Sin: return call(math_fn("sin", f16 ? ElemSize::F32 : sz, true));
+          case UnOp::Sqrt: return call(math_fn("sqrt", f16 ? ElemSize::F32 : sz, false));
+          case UnOp::Tanh: return call(math_fn("tanh", f16 ? ElemSize::F32 : sz, false));
+          case UnOp::Abs:
+            if (is_float(sz)) return call(math_fn("fabs", f16 ? ElemSize::F32 : sz, false));
+            return "(" + a + " < 0 ? -" + a + " : " + a + ")";
+        }
+        return a;
+      }
+      case Expr::BinOpE: {
+        std::string a = pexpr(e->args[0]), b = pexpr(e->args[1]);
+        ElemSize sz = e->args[0]->ty.sz;
+        switch (e->bop) {
+          case BinOp::Max: case BinOp::Min: {
+            const char* base = e->bop == BinOp::Max ? "max" : "min";
+            if (sz == ElemSize::F32) return std::string("f") + base + "f(" + a + ", " + b + ")";
+            if (sz == ElemSize::F64) return std::string("f") + base + "(" + a + ", " + b + ")";
+            if (sz == ElemSize::F16) return std::string("((_Float16)f") + base + "f((float)" + paren(a) + ", (float)" + paren(b) + "))";
+            return std::string("parpy_") + base + "<" + elem_ctype(sz) + ">(" + a + ", " + b + ")";
+          }
+          case BinOp::Atan2: return std::string(sz == ElemSize::F64 ? "atan2" : "atan2f") + "(" + a + ", " + b + ")";
+          case BinOp::Pow: return std::string(sz == ElemSize::F64 ? "pow" : "__powf") + "(" + a + ", " + b + ")";
+          default: return "(" + a + " " + cop(e->bop) + " " + b + ")";
+        }
+      }
+      case Expr::IfExpr: return "(" + pexpr(e->args[0]) + " ? " + pexpr(e->args[1]) + " : " + pexpr(e->args[2]) + ")";
+      case Expr::Convert: return "((" + std::string(elem_ctype(e->ty.sz)) + ")" + paren(pexpr(e->args[0])) + ")";
+      case Expr::Index: return pexpr(e->args[0]) + "[" + pexpr(e->args[1]) + "]";
+      case Expr::AddrOf: return "(&" + pexpr(e->args[0]) + "[" + pexpr(e->args[1]) + "])";
+      case Expr::ThreadIdx: case Expr::BlockIdx: return "((int64_t)" + idx_name(e->k, (int)e->iv) + ")";
+      case Expr::RegElem: return e->name.str() + "[" + pexpr(e->args[0]) + "]";
+      case Expr::Raw: return e->sval;
+      default: fail_rt(e->i, "Cannot print expression " + print_expr(e) + " (internal error)");
+    }
+  }
+
+  // ---------------------------------------------------------------- statements
+  static void find_reassigned(const Stmts& ss, std::set<Name>& out) {
+    for (auto& s : ss) {
+      if (s->k == Stmt::Assign && s->dst->k == Expr::Var) out.insert(s->dst->name);
+      if (s->k == Stmt::WaveReduce) out.insert(s->id);
+      find_reassigned(s->body, out);
+      find_reassigned(s->els, out);
+    }
+  }
+
+  std::string map_index(const GpuMap& m) {
+    switch (m.k) {
+      case GpuMap::Thread: return "(int)threadIdx." + std::string(1, "xyz"[m.dim]);
+      case GpuMap::Block: {
+        int64_t tot = m.dim == 0 ? kernel->grid.x : m.dim == 1 ? kernel->grid.y : kernel->grid.z;
+        std::string b = "(int)blockIdx." + std::string(1, "xyz"[m.dim]);
+        if (tot > m.n) return "((" + b + " / " + std::to_string(m.mult) + ") % " + std::to_string(m.n) + ")";
+        return b;
+      }
+      case GpuMap::ThreadBlock:
+        return "((int)blockIdx.x * " + std::to_string(m.tpb) + " + (int)threadIdx.x)";
+      default: return "0";
+    }
+  }
+
+  Interval map_index_range(const GpuMap& m) {
+    Interval r;
+    r.known = true;
+    r.lo = 0;
+    r.hi = m.k == GpuMap::ThreadBlock ? (m.n + m.tpb - 1) / m.tpb * m.tpb - 1 : m.n - 1;
+    return r;
+  }
+
+  void pfor(const S& s, int n) {
+    Interval lo = expr_range(s->lo, ranges), hi = expr_range(s->hi, ranges);
+    bool is64 = s->lo->ty.is_scalar() && s->lo->ty.sz == ElemSize::I64;
+    Interval vr;
+    if (lo.known && hi.known) {
+      vr.known = true;
+      vr.lo = s->step > 0 ? lo.lo : hi.lo + 1;
+      vr.hi = s->step > 0 ? std::max(hi.hi - 1, lo.lo) : lo.hi;
+    }
+    bool narrow = opts.opt_narrow_index && is64 && fits32(vr) && !reassigned.count(s->id);
+    // the strided increment may step past hi by up to step * N before the loop test fails
+    int64_t stride = s->step * (s->map.k == GpuMap::None ? 1 : s->map.n);
+    if (narrow && !(vr.hi + std::abs(stride) <= INT32_MAX && vr.lo - std::abs(stride) >= INT32_MIN)) narrow = false;
+    std::string vty = narrow ? "int" : elem_ctype(s->lo->ty.sz);
+    std::string v = s->id.str();
+    if (vr.known && !reassigned.count(s->id)) ranges[s->id] = vr;
+    if (narrow) narrow_vars.insert(s->id);
+    const char* cmp = s->step > 0 ? " < " : " > ";
+    std::string los = pexpr(s->lo), his = pexpr(s->hi);
+
+    if (s->map.k == GpuMap::None) {
+      if (s->unroll) os << ind(n) << "#pragma unroll\n";
+      os << ind(n) << "for (" << vty << " " << v << " = " << los << "; " << v << cmp << his << "; " << v << " += " << s->step << ") {\n";
+      pstmts(s->body, n + 2);
+      os << ind(n) << "}\n";
+      return;
+    }
+    const GpuMap& m = s->map;
+    std::string idx = map_index(m);
+    int64_t N = m.n;
+    bool const_bounds = s->lo->k == Expr::Int && s->hi->k == Expr::Int;
+    int64_t extent = 0;
+    if (const_bounds)
+      extent = s->step > 0 ? (s->hi->iv - s->lo->iv + s->step - 1) / s->step : (s->lo->iv - s->hi->iv - s->step - 1) / (-s->step);
+    int64_t launched = m.k == GpuMap::ThreadBlock ? (m.n + m.tpb - 1) / m.tpb * m.tpb : m.n;
+    std::string guard;
+    if (m.k == GpuMap::ThreadBlock && launched != m.n) guard = idx + " < " + std::to_string(m.n);
+    std::string stepmul = s->step == 1 ? "" : std::to_string(s->step) + " * ";
+    auto init = [&](const std::string& i) {
+      if (s->lo->k == Expr::Int && s->lo->iv == 0) return stepmul + i;
+      return los + " + " + stepmul + i;
+    };
+    if (const_bounds && extent <= N) {
+      // every thread (block) runs at most one iteration: no loop
+      os << ind(n) << "{\n";
+      os << ind(n + 2) << vty << " " << v << " = " << init(idx) << ";\n";
+      std::string cond;
+      if (extent < launched) cond = v + cmp + his;
+      if (!guard.empty()) cond = cond.empty() ? guard : cond + " && " + guard;
+      if (!cond.empty()) {
+        os << ind(n + 2) << "if (" << cond << ") {\n";
+        pstmts(s->body, n + 4);
+        os << ind(n + 2) << "}\n";
+      } else {
+        pstmts(s->body, n + 2);
+      }
+      os << ind(n) << "}\n";
+      return;
+    }
+    if (const_bounds && extent % N == 0 && guard.empty()) {
+      // every thread runs the same, compile-time known number of iterations
+      int64_t per = extent / N;
+      std::string k = v + "_k";
+      if (s->unroll) os << ind(n) << "#pragma unroll\n";
+      os << ind(n) << "for (int " << k << " = 0; " << k << " < " << per << "; ++" << k << ") {\n";
+      os << ind(n + 2) << vty << " " << v << " = " << init("(" + idx + " + " + k + " * " + std::to_string(N) + ")") << ";\n";
+      pstmts(s->body, n + 2);
+      os << ind(n) << "}\n";
+      return;
+    }
+    std::string cond = v + cmp + his;
+    if (!guard.empty()) cond += " && " + guard;
+    os << ind(n) << "for (" << vty << " " << v << " = " << init(idx) << "; " << cond << "; " << v << " += "
+       << (s->step * N) << ") {\n";
+    pstmts(s->body, n + 2);
+    os << ind(n) << "}\n";
+  }
+
+  void pstmt(const S& s, int n) {
+    switch (s->k) {
+      case Stmt::Def: {
+        Interval r = expr_range(s->expr, ranges);
+        bool is64 = s->ty.is_scalar() && s->ty.sz == ElemSize::I64;
+        bool fixed = !reassigned.count(s->id);
+        if (fixed && r.known) ranges[s->id] = r;
+        bool narrow = opts.opt_narrow_index && is64 && fixed && fits32(r);
+        if (narrow) narrow_vars.insert(s->id);
+        std::string rhs = pexpr(s->expr);
+        // aliases may point at read-only parameters: the qualifier is dropped, stores never go through them
+        if (!s->ty.is_scalar()) rhs = "(" + ctype(s->ty) + ")" + rhs;
+        os << ind(n) << (narrow ? std::string("int") : ctype(s->ty)) << " " << s->id.str() << " = " << rhs << ";\n";
+        break;
+      }
+      case Stmt::Assign: {
+        std::string rhs = pexpr(s->expr);
+        if (s->dst->k == Expr::Var && !s->dst->ty.is_scalar()) rhs = "(" + ctype(s->dst->ty) + ")" + rhs;
+        os << ind(n) << pexpr(s->dst) << " = " << rhs << ";\n";
+        break;
+      }
+      case Stmt::For: pfor(s, n); break;
+      case Stmt::While:
+        os << ind(n) << "while (" << pexpr(s->expr) << ") {\n";
+        pstmts(s->body, n + 2);
+        os << ind(n) << "}\n";
+        break;
+      case Stmt::If:
+        os << ind(n) << "if " << paren(pexpr(s->expr)) << " {\n";
+        pstmts(s->body, n + 2);
+        if (!s->els.empty()) {
+          os << ind(n) << "} else {\n";
+          pstmts(s->els, n + 2);
+        }
+        os << ind(n) << "}\n";
+        break;
+      case Stmt::Sync: os << ind(n) << "__syncthreads();\n"; break;
+      case Stmt::Scope:
+        os << ind(n) << "{\n";
+        pstmts(s->body, n + 2);
+        os << ind(n) << "}\n";
+        break;
+      case Stmt::WaveReduce: {
+        int64_t nwaves = std::max<int64_t>(1, s->iv / WAVE_SIZE);
+        std::string ty = elem_ctype(s->ty.sz);
+        std::string op = std::string("parpy_op_") + red_suffix(s->bop);
+        std::string v = s->id.str();
+        if (nwaves == 1) {
+          os << ind(n) << v << " = parpy_wave_reduce<" << op << ">(" << v << ");\n";
+        } else {
+          std::string slots = "parpy_red_" + std::to_string(red_sites++);
+          lds_decls.push_back("__shared__ " + ty + " " + slots + "[" + std::to_string(nwaves) + "];");
+          E ne = neutral_element(s->bop == BinOp::And ? BinOp::BitAnd : s->bop == BinOp::Or ? BinOp::BitOr : s->bop, s->ty.sz, s->i);
+          os << ind(n) << v << " = parpy_block_reduce<" << op << ", " << nwaves << ">(" << v << ", (" << ty << ")" << pexpr(ne)
+             << ", " << slots << ", " << (s->unroll ? "true" : "false") << ");\n";
+        }
+        break;
+      }
+      case Stmt::LdsDecl:
+        lds_decls.push_back("__shared__ " + std::string(elem_ctype(s->ty.sz)) + " " + s->id.str() + "[" + std::to_string(s->iv) + "];");
+        break;
+      case Stmt::RegDecl:
+        os << ind(n) << elem_ctype(s->ty.sz) << " " << s->id.str() << "[" << s->iv << "];\n";
+        break;
+      case Stmt::RawStmt: os << ind(n) << s->fname << "\n"; break;
+      default:
+        fail_rt(s->i, "Statement kind not supported in device code (internal error)");
+    }
+  }
+
+  void pstmts(const Stmts& ss, int n) {
+    for (auto& s : ss) pstmt(s, n);
+  }
+
+  std::string kernel_text(const Kernel& k) {
+    kernel = &k;
+    ranges.clear();
+    narrow_vars.clear();
+    reassigned.clear();
+    lds_decls.clear();
+    os.str("");
+    find_reassigned(k.body, reassigned);
+    pstmts(k.body, 2);
+    std::string body = os.str();
+    std::ostringstream out;
+    int64_t threads = k.block.x * k.block.y * k.block.z;
+    out << "extern \"C\" __global__ void __launch_bounds__(" << threads << ") " << k.name << "(";
+    for (size_t i = 0; i < k.params.size(); ++i) {
+      const auto& p = k.params[i];
+      out << (i ? ", " : "");
+      if (p.ty.k == Type::Pointer) out << (p.read_only ? "const " : "") << elem_ctype(p.ty.sz) << "* __restrict__ " << p.id.str();
+      else out << elem_ctype(p.ty.sz) << " " << p.id.str();
+    }
+    out << ") {\n";
+    for (auto& d : lds_decls) out << "  " << d << "\n";
+    out << body << "}\n";
+    return out.str();
+  }
+};
+
+// ---------------------------------------------------------------- host plan
+struct PlanPrinter {
+  const Program& p;
+  std::ostringstream os;
+
+  explicit PlanPrinter(const Program& prog) : p(prog) {}
+
+  std::string hexpr(const E& e) {
+    switch (e->k) {
+      case Expr::Var: return "(v " + sx_quote(e->name.str()) + ")";
+      case Expr::Int: return "(i " + std::to_string(e->iv) + ")";
+      case Expr::Float: {
+        char buf[64];
+        if (std::isinf(e->fv)) return e->fv > 0 ? "(f inf)" : "(f -inf)";
+        if (std::isnan(e->fv)) return "(f nan)";
+        snprintf(buf, sizeof buf, "%.17g", e->fv);
+        return std::string("(f ") + buf + ")";
+      }
+      case Expr::Bool: return e->bv ? "(i 1)" : "(i 0)";
+      case Expr::UnOpE: {
+        const char* n = e->uop == UnOp::Sub ? "neg" : e->uop == UnOp::Not ? "not" : e->uop == UnOp::BitNeg ? "bitneg" : nullptr;
+        if (!n) fail_rt(e->i, "Operator not supported in host code");
+        return std::string("(un ") + n + " " + hexpr(e->args[0]) + ")";
+      }
+      case Expr::BinOpE: {
+        static const std::map<BinOp, const char*> names = {
+            {BinOp::Add, "add"}, {BinOp::Sub, "sub"}, {BinOp::Mul, "mul"}, {BinOp::Div, "div"}, {BinOp::FloorDiv, "floordiv"},
+            {BinOp::Rem, "rem"}, {BinOp::And, "and"}, {BinOp::Or, "or"}, {BinOp::BitAnd, "bitand"}, {BinOp::BitOr, "bitor"},
+            {BinOp::BitXor, "bitxor"}, {BinOp::BitShl, "shl"}, {BinOp::BitShr, "shr"}, {BinOp::Eq, "eq"}, {BinOp::Neq, "neq"},
+            {BinOp::Leq, "leq"}, {BinOp::Geq, "geq"}, {BinOp::Lt, "lt"}, {BinOp::Gt, "gt"}, {BinOp::Max, "max"}, {BinOp::Min, "min"}};
+        auto it = names.find(e->bop);
+        if (it == names.end()) fail_rt(e->i, "Operator not supported in host code");
+        bool flt = e->args[0]->ty.is_scalar() && is_float(e->args[0]->ty.sz);
+        return std::string("(bin ") + it->second + (flt ? " f " : " i ") + hexpr(e->args[0]) + " " + hexpr(e->args[1]) + ")";
+      }
+      case Expr::IfExpr: return "(ite " + hexpr(e->args[0]) + " " + hexpr(e->args[1]) + " " + hexpr(e->args[2]) + ")";
+      case Expr::Convert: return std::string("(cvt ") + elem_tag(e->ty.sz) + " " + hexpr(e->args[0]) + ")";
+      case Expr::AddrOf: return "(addr " + hexpr(e->args[0]) + " " + hexpr(e->args[1]) + " " + std::to_string(elem_bytes(e->ty.sz)) + ")";
+      default: fail_rt(e->i, "Expression " + print_expr(e) + " is not supported in host code");
+    }
+  }
+
+  std::string kind_of(const Type& t) {
+    if (t.k == Type::Pointer || (t.k == Type::Tensor && !t.shape.empty())) return "ptr";
+    return elem_tag(t.sz);
+  }
+
+  void stmts(const Stmts& ss) {
+    for (auto& s : ss) {
+      switch (s->k) {
+        case Stmt::Launch: {
+          size_t idx = 0;
+          for (; idx < p.kernels.size(); ++idx)
+            if (p.kernels[idx].name == s->fname) break;
+          os << "(launch " << idx << " " << s->grid.x << " " << s->grid.y << " " << s->grid.z << " " << s->block.x << " "
+             << s->block.y << " " << s->block.z << " (args";
+          for (auto& a : s->args) os << " " << hexpr(a);
+          os << "))";
+          break;
+        }
+        case Stmt::For:
+          os << "(for " << sx_quote(s->id.str()) << " " << hexpr(s->lo) << " " << hexpr(s->hi) << " " << s->step << " (body ";
+          stmts(s->body);
+          os << "))";
+          break;
+        case Stmt::While:
+          os << "(while " << hexpr(s->expr) << " (body ";
+          stmts(s->body);
+          os << "))";
+          break;
+        case Stmt::If:
+          os << "(if " << hexpr(s->expr) << " (then ";
+          stmts(s->body);
+          os << ") (else ";
+          stmts(s->els);
+          os << "))";
+          break;
+        case Stmt::Def: os << "(def " << sx_quote(s->id.str()) << " " << kind_of(s->ty) << " " << hexpr(s->expr) << ")"; break;
+        case Stmt::Assign: os << "(set " << sx_quote(s->dst->name.str()) << " " << hexpr(s->expr) << ")"; break;
+        case Stmt::Alloc: os << "(alloc " << sx_quote(s->id.str()) << " " << s->iv * elem_bytes(s->ty.sz) << ")"; break;
+        case Stmt::Free: os << "(free " << sx_quote(s->id.str()) << ")"; break;
+        default: fail_rt(s->i, "Statement not supported in host code (internal error)");
+      }
+      os << " ";
+    }
+  }
+
+  std::string run() {
+    os << "(plan " << sx_quote(p.name) << " (params";
+    for (auto& q : p.entry_params) os << " (" << sx_quote(q.id.str()) << " ptr)";
+    os << ") (kernels";
+    for (auto& k : p.kernels) {
+      os << " (" << sx_quote(k.name) << " (params";
+      for (auto& q : k.params) os << " " << kind_of(q.ty);
+      os << "))";
+    }
+    os << ") (body ";
+    stmts(p.host);
+    os << "))";
+    return os.str();
+  }
+};
+
+// pseudo host code for the human-readable listing
+void list_host(std::ostringstream& os, const Stmts& ss, int n) {
+  std::string pad(n, ' ');
+  for (auto& s : ss) {
+    switch (s->k) {
+      case Stmt::Launch: {
+        os << pad << s->fname << "<<<dim3(" << s->grid.x << ", " << s->grid.y << ", " << s->grid.z << "), dim3(" << s->block.x
+           << ", " << s->block.y << ", " << s->block.z << "), 0, 0>>>(";
+        for (size_t i = 0; i < s->args.size(); ++i) os << (i ? ", " : "") << print_expr(s->args[i]);
+        os << ");\n";
+        break;
+      }
+      case Stmt::For:
+        os << pad << "for (int64_t " << s->id.str() << " = " << print_expr(s->lo) << "; " << s->id.str() << (s->step > 0 ? " < " : " > ")
+           << print_expr(s->hi) << "; " << s->id.str() << " += " << s->step << ") {\n";
+        list_host(os, s->body, n + 2);
+        os << pad << "}\n";
+        break;
+      case Stmt::While:
+        os << pad << "while (" << print_expr(s->expr) << ") {\n";
+        list_host(os, s->body, n + 2);
+        os << pad << "}\n";
+        break;
+      case Stmt::If:
+        os << pad << "if (" << print_expr(s->expr) << ") {\n";
+        list_host(os, s->body, n + 2);
+        if (!s->els.empty()) {
+          os << pad << "} else {\n";
+          list_host(os, s->els, n + 2);
+        }
+        os << pad << "}\n";
+        break;
+      case Stmt::Def: os << pad << "auto " << s->id.str() << " = " << print_expr(s->expr) << ";\n"; break;
+      case Stmt::Assign: os << pad << print_expr(s->dst) << " = " << print_expr(s->expr) << ";\n"; break;
+      case Stmt::Alloc:
+        os << pad << elem_ctype(s->ty.sz) << "* " << s->id.str() << " = (" << elem_ctype(s->ty.sz) << "*)parpy_alloc_buffer("
+           << s->iv * elem_bytes(s->ty.sz) << ");\n";
+        break;
+      case Stmt::Free: os << pad << "parpy_free_buffer(" << s->id.str() << ");\n"; break;
+      default: break;
+    }
+  }
+}
+
+}  // namespace
+
+std::string hip_print_device(const Program& p, const Options& opts) {
+  std::ostringstream out;
+  out << PREAMBLE;
+  for (auto& inc : p.includes) out << "#include \"" << inc << "\"\n";
+  for (auto& d : p.preamble) out << d << "\n";
+  DevicePrinter dp(opts);
+  for (auto& k : p.kernels) out << "\n" << dp.kernel_text(k);
+  return out.str();
+}
+
+std::string hip_print_plan(const Program& p) { return PlanPrinter(p).run(); }
+
+std::string hip_print_listing(const Program& p, const Options& opts) {
+  std::ostringstream out;
+  out << hip_print_device(p, opts);
+  out << "\n// host side: executed by the runtime's launch-plan interpreter (hipModuleLaunchKernel on stream 0)\n";
+  out << "extern \"C\" int32_t " << p.name << "(";
+  for (size_t i = 0; i < p.entry_params.size(); ++i)
+    out << (i ? ", " : "") << elem_ctype(p.entry_params[i].ty.sz) << "* " << p.entry_params[i].id.str();
+  out << ") {\n";
+  list_host(out, p.host, 2);
+  out << "  return 0;\n}\n";
+  return out.str();
+}
+
+}  // namespace parpy
