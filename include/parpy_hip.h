@@ -72,6 +72,14 @@ int32_t parpy_hip_plan_create(void* module, const char* plan_text, void** plan);
  * folded into the code at compile time.  Returns 0 or non-zero. */
 int32_t parpy_hip_plan_run(void* plan, void* const* args, int32_t nargs);
 
+/* Same as parpy_hip_plan_run, bracketed by HIP events recorded on the null
+ * stream right before the first and after the last launch; waits for the
+ * work to finish and returns the device time in milliseconds.  This is what
+ * the reference's benchmarks do with CUDA events around a call
+ * (benchmarks/common.py:76-89), without the Python overhead in between. */
+int32_t parpy_hip_plan_run_timed(void* plan, void* const* args, int32_t nargs,
+                                 float* elapsed_ms);
+
 /* Number of kernel launches the last run of this plan enqueued. */
 int64_t parpy_hip_plan_launch_count(void* plan);
 

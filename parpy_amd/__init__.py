@@ -52,7 +52,17 @@ def _convert_python_function_to_ir(fn, vars):
     # a decorated function is parsed with its decorator lines: they do not belong to the body
     top_map = _get_tops(None)
     info = (filepath, line_ofs, col_ofs)
-    return compiler.python_to_ir(tree, info, top_map, vars)
+    # Names are resolved the way Python itself would for `fn` -- closure cells,
+    # then the globals of the module that defines it -- with the caller's frame
+    # (what the reference consults, python/parpy/__init__.py:235-237) as fallback.
+    caller_globs, caller_locs = vars
+    globs = {**caller_globs, **getattr(fn, "__globals__", {})}
+    try:
+        nonlocals = dict(inspect.getclosurevars(fn).nonlocals)
+    except (TypeError, ValueError):
+        nonlocals = {}
+    locs = {**caller_locs, **nonlocals} if caller_locs is not caller_globs else nonlocals
+    return compiler.python_to_ir(tree, info, top_map, (globs, locs))
 
 
 def _check_kwarg(kwargs, key, expected_ty, fun_name):
@@ -144,6 +154,20 @@ def print_compiled(fun, args, opts=None):
     args = check_arguments(args, opts, False)
     top_map = _get_tops(opts.backend)
     return compiler.compile_ir(ir_ast, args, opts, top_map).listing
+
+
+def time_call(fun, *args, opts):
+    """Run the jitted function `fun` once and return the device time in milliseconds.
+
+    HIP events are recorded on the launch stream directly around the launches of
+    the compiled function (the reference's benchmarks bracket calls with CUDA
+    events, benchmarks/common.py:76-89)."""
+    from .validate import check_arguments
+    if fun not in _ir_asts:
+        raise RuntimeError("time_call expects a function decorated with parpy.jit")
+    opts = backend._resolve_backend(opts, True)
+    args = check_arguments(args, opts, True)
+    return _compile_function(_ir_asts[fun], args, opts).timed(*args)
 
 
 def external(ext_name, backend, target, header=None, parallelize=LoopPar()):

@@ -120,7 +120,19 @@ def get_wrapper(name, key, plan_text, opts):
         if status != 0:
             msg = lib.parpy_get_error_message()
             raise RuntimeError(f"{msg.decode('ascii', 'replace')}")
+    def timed(*args):
+        """Run once and return the device time in ms between the first and the last launch."""
+        flat = [x for a in args for x in _expand_arg(a)]
+        ptrs = [a._get_ptr() for a in flat if isinstance(a, Buffer) and len(a.shape) > 0]
+        arr = (ctypes.c_void_p * max(1, len(ptrs)))(*ptrs)
+        ms = ctypes.c_float()
+        status = lib.parpy_hip_plan_run_timed(plan, arr, len(ptrs), ctypes.byref(ms))
+        if status != 0:
+            raise RuntimeError(f"{lib.parpy_get_error_message().decode('ascii', 'replace')}")
+        return ms.value
+
     wrapper.__name__ = name
+    wrapper.timed = timed
     wrapper.plan = plan
     wrapper.launch_count = lambda: lib.parpy_hip_plan_launch_count(plan)
     return wrapper

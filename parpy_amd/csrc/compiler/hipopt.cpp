@@ -1,44 +1,993 @@
 // gfx950 memory code generation passes over the extracted kernels.
+//
+// The reference's backends print the loop nest as it stands
+// (src/cuda/codegen.rs:120-358): every access goes to global memory with one
+// element per thread and per iteration.  These passes restructure the kernels
+// for CDNA4's memory system instead:
+//
+//   lds_rows        rows of arrays that only one workgroup touches (a[blk, *])
+//                   and that are revisited inside an in-kernel sequential loop
+//                   live in LDS for the whole kernel (160 KB per workgroup);
+//   vectorize       thread-mapped loops with unit-stride accesses give every
+//                   thread V consecutive elements so that loads and stores
+//                   become dwordx4 / ds_*_b128;
+//   hoist_invariant loads from read-only arrays whose address depends only on
+//                   the thread's own iteration, inside a sequential loop, are
+//                   done once before the loop into per-thread registers;
+//   reg_cache       array sections that a thread alone reads and writes across
+//                   consecutive parallel loops stay in registers in between.
+//
+// Each pass can be switched off through the options (tests compare the
+// results with and without them).
+#include <algorithm>
+#include <functional>
+
 #include "passes.hpp"
 
 namespace parpy {
 
 namespace {
 
-// A pointer parameter is read-only when nothing in the kernel stores through
-// it, directly or through a local alias initialised from it.
-void mark_read_only(Kernel& k) {
-  std::set<Name> written;
-  std::map<Name, std::set<Name>> alias_of;  // local pointer -> parameters it may point into
-  std::function<void(const E&, std::set<Name>&)> bases = [&](const E& e, std::set<Name>& out) {
-    if (!e) return;
-    if (e->k == Expr::Var) {
-      auto it = alias_of.find(e->name);
-      if (it != alias_of.end()) out.insert(it->second.begin(), it->second.end());
-      else out.insert(e->name);
-      return;
-    }
-    if (e->k == Expr::AddrOf || e->k == Expr::Index) { bases(e->args[0], out); return; }
-    if (e->k == Expr::IfExpr) { bases(e->args[1], out); bases(e->args[2], out); }
-  };
-  // two sweeps so that aliases assigned after their first use inside loops are seen
-  for (int sweep = 0; sweep < 2; ++sweep) {
-    visit_stmts(k.body, [&](const S& s) {
-      if (s->k == Stmt::Def && (s->ty.is_array() || s->ty.is_pointer())) bases(s->expr, alias_of[s->id]);
-      if (s->k == Stmt::Assign && s->dst->k == Expr::Var && (s->dst->ty.is_array() || s->dst->ty.is_pointer()))
-        bases(s->expr, alias_of[s->dst->name]);
-      if (s->k == Stmt::Assign && s->dst->k == Expr::Index) bases(s->dst->args[0], written);
-    });
-  }
-  for (auto& p : k.params) p.read_only = p.ty.is_pointer() && !written.count(p.id);
+using StmtP = std::shared_ptr<Stmt>;
+StmtP clone(const S& s) { return std::make_shared<Stmt>(*s); }
+
+constexpr int64_t LDS_BUDGET_BYTES = 160 * 1024 - 4096;  // leave room for reduction slots
+
+bool mentions(const E& e, const Name& v) {
+  bool m = false;
+  visit_exprs(e, [&](const E& x) { if (x->k == Expr::Var && x->name == v) m = true; });
+  return m;
 }
+
+bool has_load(const E& e) {
+  bool m = false;
+  visit_exprs(e, [&](const E& x) { if (x->k == Expr::Index || x->k == Expr::AddrOf || x->k == Expr::RegElem) m = true; });
+  return m;
+}
+
+// idx == rest + d with rest free of d
+bool affine_unit(const E& idx, const Name& d, E* rest) {
+  if (idx->k == Expr::Var && idx->name == d) { *rest = mk_int(0, idx->ty.sz); return true; }
+  if (idx->k == Expr::BinOpE && (idx->bop == BinOp::Add || idx->bop == BinOp::Sub)) {
+    E r;
+    if (affine_unit(idx->args[0], d, &r) && !mentions(idx->args[1], d)) {
+      *rest = fold_expr(mk_binop(idx->bop, r, idx->args[1], idx->ty));
+      return true;
+    }
+    if (idx->bop == BinOp::Add && affine_unit(idx->args[1], d, &r) && !mentions(idx->args[0], d)) {
+      *rest = fold_expr(mk_binop(BinOp::Add, idx->args[0], r, idx->ty));
+      return true;
+    }
+  }
+  return false;
+}
+
+int64_t const_extent(const S& loop) {
+  if (loop->lo->k != Expr::Int || loop->hi->k != Expr::Int || loop->step <= 0) return -1;
+  return (loop->hi->iv - loop->lo->iv + loop->step - 1) / loop->step;
+}
+
+bool thread_mapped(const S& s) { return s->k == Stmt::For && s->map.k == GpuMap::Thread; }
+
+// iterations every thread runs in a thread-mapped loop, when that is a compile-time constant
+int64_t per_thread_trips(const S& loop) {
+  int64_t e = const_extent(loop);
+  if (e <= 0 || loop->map.n <= 0 || e % loop->map.n != 0) return -1;
+  return e / loop->map.n;
+}
+
+// the per-thread iteration counter of a mapped loop as the printer names it
+E counter_var(const S& loop, ElemSize isz) {
+  if (per_thread_trips(loop) == 1) return mk_int(0, isz);
+  return mk_var(Name{loop->id.str() + "_k", 0}, Type::scalar(isz));
+}
+
+E subst_vars(const E& e, const std::map<Name, E>& m) {
+  if (!e) return e;
+  if (e->k == Expr::Var) {
+    auto it = m.find(e->name);
+    return it == m.end() ? e : it->second;
+  }
+  return map_children(e, [&](const E& c) { return subst_vars(c, m); });
+}
+
+template <class F> E rewrite_expr(const E& e, F f) {  // bottom-up rewrite
+  if (!e) return e;
+  E r = map_children(e, [&](const E& c) { return rewrite_expr(c, f); });
+  return f(r);
+}
+
+template <class F> Stmts rewrite_stmts(const Stmts& ss, F f) {  // f : E -> E applied to every expression, deep
+  Stmts out;
+  for (auto& s : ss) {
+    auto r = std::const_pointer_cast<Stmt>(std::static_pointer_cast<const Stmt>(map_exprs(s, [&](const E& e) { return rewrite_expr(e, f); })));
+    r->body = rewrite_stmts(s->body, f);
+    r->els = rewrite_stmts(s->els, f);
+    out.push_back(r);
+  }
+  return out;
+}
+
+struct Pass {
+  Kernel& k;
+  const Options& opts;
+  NameGen& gen;
+  ElemSize isz;
+
+  Pass(Kernel& kernel, const Options& o, NameGen& g) : k(kernel), opts(o), gen(g), isz(o.int_size()) {}
+
+  std::set<Name> param_names() const {
+    std::set<Name> r;
+    for (auto& p : k.params) r.insert(p.id);
+    return r;
+  }
+
+  // ================================================================ unswitching of array aliases
+  // `src = a; dst = b; if (c) { src = b; dst = a; } <rest>` becomes
+  // `if (c) { <rest with src=b, dst=a> } else { <rest with src=a, dst=b> }`.
+  // Every access then names its array directly, which is what lets the target
+  // compiler prove that loads from one buffer do not alias stores to the other
+  // (it merges and reorders LDS accesses accordingly) and what the LDS and
+  // register passes below analyse.  The condition is evaluated where it was.
+  struct Unswitch {
+    bool failed = false;
+    int clones = 0;
+
+    static bool is_alias_type(const Type& t) { return t.k == Type::Tensor ? !t.shape.empty() : t.k == Type::Pointer; }
+
+    E resolve(const E& e, const std::map<Name, E>& env) {
+      if (e->k == Expr::Var) {
+        auto it = env.find(e->name);
+        return it == env.end() ? e : it->second;
+      }
+      return e;
+    }
+
+    // a statement that does nothing but (conditionally) repoint aliases
+    bool pure_select(const S& s, const std::map<Name, E>& env) {
+      if (s->k == Stmt::Assign) return s->dst->k == Expr::Var && env.count(s->dst->name) && s->expr->k == Expr::Var;
+      if (s->k == Stmt::If) {
+        if (s->body.empty() && s->els.empty()) return false;
+        for (auto& c : s->body) if (!pure_select(c, env)) return false;
+        for (auto& c : s->els) if (!pure_select(c, env)) return false;
+        return true;
+      }
+      return false;
+    }
+
+    void apply_selects(const Stmts& ss, std::map<Name, E>& env) {
+      for (auto& s : ss)
+        if (s->k == Stmt::Assign) env[s->dst->name] = resolve(s->expr, env);
+    }
+
+    bool has_nested_if(const Stmts& ss) {
+      for (auto& s : ss)
+        if (s->k == Stmt::If) return true;
+      return false;
+    }
+
+    E subst(const E& e, const std::map<Name, E>& env) {
+      if (!e) return e;
+      if (e->k == Expr::Var) {
+        auto it = env.find(e->name);
+        return it == env.end() ? e : it->second;
+      }
+      return map_children(e, [&](const E& c) { return subst(c, env); });
+    }
+
+    Stmts run(const Stmts& ss, size_t from, std::map<Name, E> env) {
+      Stmts out;
+      for (size_t i = from; i < ss.size(); ++i) {
+        const S& s = ss[i];
+        if (s->k == Stmt::Def && is_alias_type(s->ty) && s->expr->k == Expr::Var) {
+          env[s->id] = resolve(s->expr, env);
+          continue;
+        }
+        if (s->k == Stmt::Assign && s->dst->k == Expr::Var && env.count(s->dst->name)) {
+          if (s->expr->k != Expr::Var) { failed = true; return out; }
+          env[s->dst->name] = resolve(s->expr, env);
+          continue;
+        }
+        if (s->k == Stmt::If && !env.empty() && pure_select(s, env)) {
+          if (has_nested_if(s->body) || has_nested_if(s->els) || ++clones > 4) { failed = true; return out; }
+          std::map<Name, E> et = env, ee = env;
+          apply_selects(s->body, et);
+          apply_selects(s->els, ee);
+          auto n = clone(s);
+          n->expr = subst(s->expr, env);
+          n->body = run(ss, i + 1, et);
+          n->els = run(ss, i + 1, ee);
+          out.push_back(n);
+          return out;
+        }
+        // an alias assigned anywhere else (inside a loop body, say) cannot be tracked
+        bool bad = false;
+        std::function<void(const Stmts&)> check = [&](const Stmts& b) {
+          for (auto& c : b) {
+            if (c->k == Stmt::Assign && c->dst->k == Expr::Var && env.count(c->dst->name)) bad = true;
+            check(c->body);
+            check(c->els);
+          }
+        };
+        check(s->body);
+        check(s->els);
+        if (bad) { failed = true; return out; }
+        auto n = std::const_pointer_cast<Stmt>(std::static_pointer_cast<const Stmt>(map_exprs(s, [&](const E& e) { return subst(e, env); })));
+        n->body = run(s->body, 0, env);
+        n->els = run(s->els, 0, env);
+        out.push_back(n);
+      }
+      return out;
+    }
+  };
+
+  void unswitch_aliases() {
+    bool any = false;
+    visit_stmts(k.body, [&](const S& s) { if (s->k == Stmt::Def && Unswitch::is_alias_type(s->ty)) any = true; });
+    if (!any) return;
+    Unswitch u;
+    Stmts nb = u.run(k.body, 0, {});
+    if (!u.failed) k.body = nb;
+  }
+
+  // ================================================================ LDS rows
+  struct ArrayInfo {
+    bool ok = true;
+    int64_t rowlen = 0;
+    ElemSize sz = ElemSize::F32;
+    bool in_seq_loop = false;
+    bool written = false;
+    bool accessed = false;
+  };
+
+  void lds_rows() {
+    if (k.body.size() != 1 || k.body[0]->k != Stmt::For || k.body[0]->map.k != GpuMap::Block) return;
+    const S root = k.body[0];
+    int64_t ext = const_extent(root);
+    if (ext <= 0 || ext > root->map.n) return;  // a block must own exactly one value of the root variable
+    if (k.block.y != 1 || k.block.z != 1) return;
+    const Name r = root->id;
+
+    std::map<Name, ArrayInfo> info;
+    for (auto& p : k.params)
+      if (p.ty.is_pointer()) info[p.id] = ArrayInfo();
+    std::map<Name, std::set<Name>> alias;  // local -> parameters it may point to
+
+    std::function<bool(const E&, std::set<Name>&)> sources = [&](const E& e, std::set<Name>& out) -> bool {
+      if (e->k == Expr::Var) {
+        if (info.count(e->name)) { out.insert(e->name); return true; }
+        auto it = alias.find(e->name);
+        if (it != alias.end()) { out.insert(it->second.begin(), it->second.end()); return true; }
+        return false;
+      }
+      if (e->k == Expr::IfExpr) return sources(e->args[1], out) && sources(e->args[2], out);
+      return false;
+    };
+    // aliases first (two sweeps reach a fixed point for loop-carried selects)
+    for (int sweep = 0; sweep < 2; ++sweep)
+      visit_stmts(k.body, [&](const S& s) {
+        if (s->k == Stmt::Def && !s->ty.is_scalar()) { std::set<Name> src; if (sources(s->expr, src)) alias[s->id].insert(src.begin(), src.end()); }
+        if (s->k == Stmt::Assign && s->dst->k == Expr::Var && !s->dst->ty.is_scalar()) {
+          std::set<Name> src;
+          if (sources(s->expr, src)) alias[s->dst->name].insert(src.begin(), src.end());
+        }
+      });
+
+    // every use of an array (or alias) must be a two-dimensional access a[r, e]
+    std::function<void(const E&, bool, bool)> scan = [&](const E& e, bool in_seq, bool is_store_dst) {
+      if (!e) return;
+      if (e->k == Expr::Index || e->k == Expr::AddrOf) {
+        std::set<Name> src;
+        if (sources(e->args[0], src)) {
+          bool row = e->k == Expr::Index && e->dim_idx.size() == 2 && e->dim_idx[0]->k == Expr::Var && e->dim_idx[0]->name == r;
+          for (auto& a : src) {
+            ArrayInfo& ai = info[a];
+            if (!row) { ai.ok = false; continue; }
+            int64_t len = e->dim_shape[1];
+            if (ai.accessed && (ai.rowlen != len || ai.sz != e->ty.sz)) ai.ok = false;
+            ai.accessed = true;
+            ai.rowlen = len;
+            ai.sz = e->ty.sz;
+            ai.in_seq_loop = ai.in_seq_loop || in_seq;
+            ai.written = ai.written || is_store_dst;
+          }
+          scan(e->args[1], in_seq, false);
+          for (auto& d : e->dim_idx) scan(d, in_seq, false);
+          return;
+        }
+      }
+      if (e->k == Expr::Var) {
+        // a bare use of an array value that is not an alias definition (handled by the caller)
+        std::set<Name> src;
+        if (!e->ty.is_scalar() && sources(e, src))
+          for (auto& a : src) info[a].ok = false;
+        return;
+      }
+      for (auto& a : e->args) scan(a, in_seq, false);
+    };
+    std::function<void(const Stmts&, bool)> scan_stmts = [&](const Stmts& ss, bool in_seq) {
+      for (auto& s : ss) {
+        bool alias_def = (s->k == Stmt::Def && !s->ty.is_scalar()) ||
+                         (s->k == Stmt::Assign && s->dst->k == Expr::Var && !s->dst->ty.is_scalar());
+        if (alias_def) {
+          std::set<Name> src;
+          if (!sources(s->expr, src)) scan(s->expr, in_seq, false);
+        } else {
+          if (s->dst) scan(s->dst, in_seq, s->k == Stmt::Assign);
+          if (s->expr) scan(s->expr, in_seq, false);
+        }
+        if (s->lo) scan(s->lo, in_seq, false);
+        if (s->hi) scan(s->hi, in_seq, false);
+        for (auto& a : s->args) scan(a, in_seq, false);
+        bool seq = in_seq || (s->k == Stmt::For && s->map.k == GpuMap::None) || s->k == Stmt::While;
+        scan_stmts(s->body, seq);
+        scan_stmts(s->els, seq);
+      }
+    };
+    scan_stmts(root->body, false);
+
+    // arrays reachable through a common alias are promoted together or not at all
+    bool changed = true;
+    while (changed) {
+      changed = false;
+      for (auto& kv : alias) {
+        bool all_ok = true, any_seq = false, any_written = false;
+        int64_t len = -1;
+        ElemSize sz = ElemSize::F32;
+        for (auto& a : kv.second) {
+          const ArrayInfo& ai = info[a];
+          if (!ai.ok || !ai.accessed) { if (!ai.ok) all_ok = false; continue; }
+          if (len >= 0 && (len != ai.rowlen || sz != ai.sz)) all_ok = false;
+          len = ai.rowlen;
+          sz = ai.sz;
+          any_seq = any_seq || ai.in_seq_loop;
+          any_written = any_written || ai.written;
+        }
+        for (auto& a : kv.second) {
+          ArrayInfo& ai = info[a];
+          if (!all_ok && ai.ok) { ai.ok = false; changed = true; }
+          if (all_ok && len >= 0) {
+            if (!ai.accessed) { ai.accessed = true; ai.rowlen = len; ai.sz = sz; changed = true; }
+            if (any_seq && !ai.in_seq_loop) { ai.in_seq_loop = true; changed = true; }
+            if (any_written && !ai.written) { ai.written = true; changed = true; }
+          }
+        }
+      }
+    }
+
+    // choose what fits
+    std::map<Name, Name> lds_name;
+    int64_t used = 0;
+    for (auto& p : k.params) {
+      auto it = info.find(p.id);
+      if (it == info.end()) continue;
+      const ArrayInfo& ai = it->second;
+      if (!ai.ok || !ai.accessed || !ai.in_seq_loop || !ai.written) continue;  // read-only tables stream better from L2
+      int64_t bytes = ai.rowlen * elem_bytes(ai.sz);
+      if (used + bytes > LDS_BUDGET_BYTES) { used = LDS_BUDGET_BYTES + 1; break; }
+      used += bytes;
+      lds_name[p.id] = gen.fresh("lds_" + p.id.s);
+    }
+    if (used > LDS_BUDGET_BYTES || lds_name.empty()) return;
+    // an alias must not mix promoted and non-promoted arrays
+    for (auto& kv : alias) {
+      size_t n = 0;
+      for (auto& a : kv.second) n += lds_name.count(a);
+      if (n != 0 && n != kv.second.size()) return;
+    }
+    std::set<Name> lds_alias;
+    for (auto& kv : alias)
+      if (!kv.second.empty() && lds_name.count(*kv.second.begin())) lds_alias.insert(kv.first);
+
+    auto lds_var = [&](const Name& a, const Info& i) { return mk_var(lds_name.at(a), Type::pointer(info[a].sz, Mem::LDS), i); };
+    auto rw = [&](const E& e) -> E {
+      if (e->k == Expr::Index && e->args[0]->k == Expr::Var) {
+        const Name& b = e->args[0]->name;
+        if (lds_name.count(b)) {
+          auto n = std::make_shared<Expr>(*e);
+          n->args = {lds_var(b, e->i), e->dim_idx[1]};
+          n->dim_idx.clear();
+          n->dim_shape.clear();
+          return n;
+        }
+        if (lds_alias.count(b)) {
+          auto n = std::make_shared<Expr>(*e);
+          n->args = {mk_var(b, Type::pointer(e->ty.sz, Mem::LDS), e->i), e->dim_idx[1]};
+          n->dim_idx.clear();
+          n->dim_shape.clear();
+          return n;
+        }
+      }
+      return e;
+    };
+    Stmts body = rewrite_stmts(root->body, rw);
+    // alias definitions now select between LDS arrays
+    std::function<E(const E&)> to_lds = [&](const E& e) -> E {
+      if (e->k == Expr::Var && lds_name.count(e->name)) return lds_var(e->name, e->i);
+      if (e->k == Expr::Var && lds_alias.count(e->name)) return mk_var(e->name, Type::pointer(e->ty.sz, Mem::LDS), e->i);
+      if (e->k == Expr::IfExpr) {
+        E a = to_lds(e->args[1]), b = to_lds(e->args[2]);
+        return mk_ifexpr(e->args[0], a, b, a->ty, e->i);
+      }
+      return e;
+    };
+    std::function<Stmts(const Stmts&)> fix_alias = [&](const Stmts& ss) {
+      Stmts out;
+      for (auto& s : ss) {
+        auto n = clone(s);
+        if (s->k == Stmt::Def && lds_alias.count(s->id)) {
+          n->expr = to_lds(s->expr);
+          n->ty = n->expr->ty;
+        } else if (s->k == Stmt::Assign && s->dst->k == Expr::Var && lds_alias.count(s->dst->name)) {
+          n->expr = to_lds(s->expr);
+          n->dst = mk_var(s->dst->name, n->expr->ty, s->dst->i);
+        }
+        n->body = fix_alias(s->body);
+        n->els = fix_alias(s->els);
+        out.push_back(n);
+      }
+      return out;
+    };
+    body = fix_alias(body);
+
+    // prologue: bring the rows in; epilogue: write them back
+    Type ity = Type::scalar(isz);
+    auto copy_loop = [&](const Name& a, bool to_lds_dir) {
+      const ArrayInfo& ai = info[a];
+      Name e = gen.fresh("e");
+      E ev = mk_var(e, ity);
+      E rv = mk_var(r, ity);
+      E flat = fold_expr(mk_binop(BinOp::Add, mk_binop(BinOp::Mul, rv, mk_int(ai.rowlen, isz), ity), ev, ity));
+      Type elem = Type::scalar(ai.sz);
+      E g = mk_index(mk_var(a, Type::pointer(ai.sz)), flat, elem);
+      E l = mk_index(lds_var(a, Info()), ev, elem);
+      LoopPar par;
+      par.nthreads = k.block.x;
+      auto loop = std::const_pointer_cast<Stmt>(std::static_pointer_cast<const Stmt>(
+          mk_for(e, mk_int(0, isz), mk_int(ai.rowlen, isz), 1, {to_lds_dir ? mk_assign(l, g) : mk_assign(g, l)}, par)));
+      loop->map.k = GpuMap::Thread;
+      loop->map.dim = 0;
+      loop->map.n = k.block.x;
+      return S(loop);
+    };
+    Stmts nb;
+    for (auto& kv : lds_name) {
+      auto d = std::make_shared<Stmt>();
+      d->k = Stmt::LdsDecl;
+      d->id = kv.second;
+      d->ty = Type::scalar(info[kv.first].sz);
+      d->iv = info[kv.first].rowlen;
+      nb.push_back(d);
+    }
+    for (auto& kv : lds_name) nb.push_back(copy_loop(kv.first, true));
+    nb.push_back(mk_sync());
+    for (auto& s : body) nb.push_back(s);
+    nb.push_back(mk_sync());
+    for (auto& kv : lds_name)
+      if (info[kv.first].written) nb.push_back(copy_loop(kv.first, false));
+    auto nr = clone(root);
+    nr->body = nb;
+    k.body = {nr};
+    int64_t total = 0;
+    for (auto& kv : lds_name) total += info[kv.first].rowlen * elem_bytes(info[kv.first].sz);
+    k.lds_bytes += total;
+  }
+
+  // ================================================================ vectorised iteration remap
+  int vector_width(const S& loop) {
+    int v = 0;
+    std::function<void(const E&)> scan = [&](const E& e) {
+      visit_exprs(e, [&](const E& x) {
+        if (x->k != Expr::Index) return;
+        E rest;
+        if (!affine_unit(x->args[1], loop->id, &rest)) return;
+        int w = elem_bytes(x->ty.sz) == 8 ? 2 : elem_bytes(x->ty.sz) == 4 ? 4 : 0;
+        if (w == 0) return;
+        v = v == 0 ? w : std::min(v, w);
+      });
+    };
+    visit_stmts(loop->body, [&](const S& s) { scan(s->dst); scan(s->expr); scan(s->lo); scan(s->hi); });
+    return v;
+  }
+
+  Stmts vectorize(const Stmts& ss) {
+    Stmts out;
+    for (auto& s : ss) {
+      bool done = false;
+      if (thread_mapped(s) && s->step == 1 && s->lo->k == Expr::Int && s->hi->k == Expr::Int) {
+        int64_t extent = const_extent(s);
+        int V = vector_width(s);
+        bool nested = false;
+        visit_stmts(s->body, [&](const S& c) { if (c->k == Stmt::For && c->map.k != GpuMap::None) nested = true; });
+        if (V > 0 && !nested && extent > 0 && extent % (s->map.n * V) == 0) {
+          Type ity = Type::scalar(isz);
+          Name q = gen.fresh(s->id.s + "_q"), u = gen.fresh(s->id.s + "_u");
+          E d = fold_expr(mk_binop(BinOp::Add, s->lo,
+                                   mk_binop(BinOp::Add, mk_binop(BinOp::Mul, mk_var(q, ity), mk_int(V, isz), ity), mk_var(u, ity), ity), ity));
+          Stmts ib;
+          ib.push_back(mk_def(s->id, ity, d, s->i));
+          for (auto& b : s->body) ib.push_back(b);
+          auto inner = std::const_pointer_cast<Stmt>(std::static_pointer_cast<const Stmt>(
+              mk_for(u, mk_int(0, isz), mk_int(V, isz), 1, ib, LoopPar(), s->i)));
+          inner->unroll = true;
+          auto outer = clone(s);
+          outer->id = q;
+          outer->lo = mk_int(0, isz);
+          outer->hi = mk_int(extent / V, isz);
+          outer->body = {S(inner)};
+          out.push_back(outer);
+          done = true;
+        }
+      }
+      if (done) continue;
+      auto r = clone(s);
+      r->body = vectorize(s->body);
+      r->els = vectorize(s->els);
+      out.push_back(r);
+    }
+    return out;
+  }
+
+  // ================================================================ hoisting of thread-private invariant loads
+  // The iteration structure of a thread-mapped loop: the mapped loop itself and,
+  // after vectorisation, the unrolled inner loop over the V consecutive elements.
+  struct IterSpace {
+    S outer;                 // thread-mapped loop
+    S inner;                 // unrolled element loop, or null
+    E slot;                  // per-thread iteration number (register array index)
+    int64_t slots = 0;
+    const Stmts* body = nullptr;  // innermost body
+  };
+
+  bool iter_space(const S& loop, IterSpace* is) {
+    int64_t per = per_thread_trips(loop);
+    if (per <= 0) return false;
+    is->outer = loop;
+    Type ity = Type::scalar(isz);
+    E kq = counter_var(loop, isz);
+    if (loop->body.size() == 1 && loop->body[0]->k == Stmt::For && loop->body[0]->unroll &&
+        loop->body[0]->map.k == GpuMap::None && const_extent(loop->body[0]) > 0 && loop->body[0]->lo->k == Expr::Int &&
+        loop->body[0]->lo->iv == 0) {
+      is->inner = loop->body[0];
+      int64_t V = const_extent(is->inner);
+      is->slots = per * V;
+      is->slot = fold_expr(mk_binop(BinOp::Add, mk_binop(BinOp::Mul, kq, mk_int(V, isz), ity), mk_var(is->inner->id, ity), ity));
+      is->body = &is->inner->body;
+    } else {
+      is->slots = per;
+      is->slot = kq;
+      is->body = &loop->body;
+    }
+    return true;
+  }
+
+  std::set<Name> written_arrays() {
+    std::set<Name> w;
+    visit_stmts(k.body, [&](const S& s) {
+      if (s->k == Stmt::Assign && s->dst->k == Expr::Index) {
+        visit_exprs(s->dst->args[0], [&](const E& x) { if (x->k == Expr::Var) w.insert(x->name); });
+      }
+    });
+    return w;
+  }
+
+  struct Hoisted { E load; Name reg; ElemSize sz; };
+
+  int64_t reg_budget() const {
+    if (opts.reg_budget > 0) return opts.reg_budget;
+    int64_t threads = k.block.x * k.block.y * k.block.z;
+    // a 1024-thread block leaves 128 VGPRs per lane; 96 cached values plus the
+    // working set still fit without spilling (measured on the HMM kernels)
+    return threads <= 256 ? 192 : threads <= 512 ? 128 : 96;
+  }
+
+  // hoist out of the sequential loop `seq` (a statement of `parent`)
+  Stmts hoist_from_seq_loop(const S& seq, int64_t* budget) {
+    std::set<Name> params = param_names();
+    std::set<Name> written = written_arrays();
+    std::set<Name> reassigned;
+    visit_stmts(k.body, [&](const S& s) { if (s->k == Stmt::Assign && s->dst->k == Expr::Var) reassigned.insert(s->dst->name); });
+
+    Stmts pre;  // statements to run before the sequential loop
+    std::function<Stmts(const Stmts&)> walk = [&](const Stmts& ss) -> Stmts {
+      Stmts out;
+      for (auto& s : ss) {
+        IterSpace is;
+        if (thread_mapped(s) && iter_space(s, &is)) {
+          // definitions inside the body that are pure functions of the iteration
+          std::map<Name, E> defs;
+          std::set<Name> iter_vars{s->id};
+          if (is.inner) iter_vars.insert(is.inner->id);
+          std::function<void(const Stmts&)> collect_defs = [&](const Stmts& b) {
+            for (auto& c : b) {
+              if (c->k == Stmt::Def && c->ty.is_scalar() && !reassigned.count(c->id) && !has_load(c->expr)) {
+                E e = subst_vars(c->expr, defs);
+                bool pure = true;
+                visit_exprs(e, [&](const E& x) { if (x->k == Expr::Var && !iter_vars.count(x->name)) pure = false; });
+                if (pure) defs[c->id] = e;
+              }
+              collect_defs(c->body);
+              collect_defs(c->els);
+            }
+          };
+          collect_defs(*is.body);
+          RangeEnv env;
+          {
+            Interval r;
+            r.known = true;
+            r.lo = s->lo->iv;
+            r.hi = s->hi->iv - 1;
+            env[s->id] = r;
+            if (is.inner) { Interval u; u.known = true; u.lo = 0; u.hi = const_extent(is.inner) - 1; env[is.inner->id] = u; }
+          }
+          std::vector<Hoisted> hoisted;
+          auto try_hoist = [&](const E& e) -> E {
+            if (e->k != Expr::Index || e->args[0]->k != Expr::Var) return e;
+            const Name& base = e->args[0]->name;
+            if (!params.count(base) || written.count(base) || e->dim_shape.empty()) return e;
+            E idx = fold_expr(subst_vars(e->args[1], defs));
+            bool pure = true;
+            visit_exprs(idx, [&](const E& x) {
+              if (x->k == Expr::Var && !iter_vars.count(x->name)) pure = false;
+              if (x->k == Expr::Index || x->k == Expr::RegElem || x->k == Expr::ThreadIdx || x->k == Expr::BlockIdx) pure = false;
+            });
+            if (!pure) return e;
+            int64_t numel = 1;
+            for (auto d : e->dim_shape) numel *= d;
+            Interval r = expr_range(idx, env);
+            if (!r.known || r.lo < 0 || r.hi >= numel) return e;  // the load is executed unconditionally once hoisted
+            for (auto& h : hoisted)
+              if (h.load->args[0]->name == base && expr_eq(h.load->args[1], idx)) {
+                auto re = std::make_shared<Expr>();
+                re->k = Expr::RegElem;
+                re->ty = e->ty;
+                re->name = h.reg;
+                re->args = {is.slot};
+                return re;
+              }
+            int64_t cost = is.slots * std::max(1, elem_bytes(e->ty.sz) / 4);
+            if (*budget < cost) return e;
+            *budget -= cost;
+            Hoisted h;
+            auto ld = std::make_shared<Expr>(*e);
+            ld->args = {e->args[0], idx};
+            h.load = ld;
+            h.reg = gen.fresh("inv_" + base.s);
+            h.sz = e->ty.sz;
+            hoisted.push_back(h);
+            auto re = std::make_shared<Expr>();
+            re->k = Expr::RegElem;
+            re->ty = e->ty;
+            re->name = h.reg;
+            re->args = {is.slot};
+            return re;
+          };
+          Stmts nbody = rewrite_stmts(*is.body, try_hoist);
+          if (hoisted.empty()) { out.push_back(s); continue; }
+          // loop nest that fills the registers, with the same thread mapping
+          std::map<Name, Name> ren;
+          Name nq = gen.fresh(s->id.s);
+          ren[s->id] = nq;
+          Name nu;
+          if (is.inner) { nu = gen.fresh(is.inner->id.s); ren[is.inner->id] = nu; }
+          std::map<Name, E> rv;
+          Type ity = Type::scalar(isz);
+          for (auto& kv : ren) rv[kv.first] = mk_var(kv.second, ity);
+          auto fill_outer = clone(s);
+          fill_outer->id = nq;
+          fill_outer->unroll = true;
+          // the counter of the fill loop has its own name: rebuild the slot expression for it
+          E fill_slot;
+          {
+            E kq = counter_var(fill_outer, isz);
+            if (is.inner) {
+              int64_t V = const_extent(is.inner);
+              fill_slot = fold_expr(mk_binop(BinOp::Add, mk_binop(BinOp::Mul, kq, mk_int(V, isz), ity), mk_var(nu, ity), ity));
+            } else {
+              fill_slot = kq;
+            }
+          }
+          Stmts fills;
+          for (auto& h : hoisted) {
+            auto d = std::make_shared<Stmt>();
+            d->k = Stmt::RegDecl;
+            d->id = h.reg;
+            d->ty = Type::scalar(h.sz);
+            d->iv = is.slots;
+            pre.push_back(d);
+            auto re = std::make_shared<Expr>();
+            re->k = Expr::RegElem;
+            re->ty = Type::scalar(h.sz);
+            re->name = h.reg;
+            re->args = {fill_slot};
+            auto ld = std::make_shared<Expr>(*h.load);
+            ld->args = {h.load->args[0], subst_vars(h.load->args[1], rv)};
+            ld->dim_idx.clear();
+            fills.push_back(mk_assign(re, ld));
+          }
+          if (is.inner) {
+            auto fi = clone(is.inner);
+            fi->id = nu;
+            fi->body = fills;
+            fill_outer->body = {S(fi)};
+          } else {
+            fill_outer->body = fills;
+          }
+          pre.push_back(fill_outer);
+          // the loop itself must be fully unrolled so that the arrays stay in registers
+          auto ns = clone(s);
+          ns->unroll = true;
+          if (is.inner) {
+            auto ni = clone(is.inner);
+            ni->body = nbody;
+            ns->body = {S(ni)};
+          } else {
+            ns->body = nbody;
+          }
+          out.push_back(ns);
+          continue;
+        }
+        auto r = clone(s);
+        r->body = walk(s->body);
+        r->els = walk(s->els);
+        out.push_back(r);
+      }
+      return out;
+    };
+    auto nseq = clone(seq);
+    nseq->body = walk(seq->body);
+    pre.push_back(nseq);
+    return pre;
+  }
+
+  Stmts hoist_invariant(const Stmts& ss, int64_t* budget, bool in_seq) {
+    Stmts out;
+    for (auto& s : ss) {
+      bool seq = (s->k == Stmt::For && s->map.k == GpuMap::None && !s->unroll) || s->k == Stmt::While;
+      if (seq && !in_seq) {
+        for (auto& r : hoist_from_seq_loop(s, budget)) out.push_back(r);
+        continue;
+      }
+      auto r = clone(s);
+      r->body = hoist_invariant(s->body, budget, in_seq);
+      r->els = hoist_invariant(s->els, budget, in_seq);
+      out.push_back(r);
+    }
+    return out;
+  }
+
+  // ================================================================ register caching across parallel loops
+  // Consecutive thread-mapped loops with the same iteration structure give each
+  // thread the same elements every time.  An array that is only ever accessed
+  // as a[inv + d] inside those loops (d the loop's element) is therefore private
+  // to the thread between them: it is read from memory once, kept in registers
+  // across the loops (and the block synchronisations between them), and written
+  // back by the last loop that stores to it.
+  void reg_cache(int64_t* budget) {
+    if (k.body.size() != 1 || k.body[0]->k != Stmt::For || k.body[0]->map.k != GpuMap::Block) return;
+    const S root = k.body[0];
+    struct Cand { size_t pos; S loop; IterSpace is; Name elem; };
+    std::vector<Cand> cands;
+    for (size_t pos = 0; pos < root->body.size(); ++pos) {
+      const S& s = root->body[pos];
+      Cand c;
+      if (!thread_mapped(s) || !iter_space(s, &c.is)) continue;
+      c.pos = pos;
+      c.loop = s;
+      // element variable: the loop variable, or the definition at the head of the unrolled element loop
+      if (c.is.inner) {
+        if (c.is.body->empty() || (*c.is.body)[0]->k != Stmt::Def) continue;
+        c.elem = (*c.is.body)[0]->id;
+      } else {
+        c.elem = s->id;
+      }
+      cands.push_back(c);
+    }
+    if (cands.size() < 2) return;
+    // loops must agree on extent, mapping and element width
+    auto same = [&](const Cand& a, const Cand& b) {
+      return const_extent(a.loop) == const_extent(b.loop) && a.loop->map.n == b.loop->map.n && a.is.slots == b.is.slots &&
+             a.loop->lo->iv == b.loop->lo->iv && (a.is.inner != nullptr) == (b.is.inner != nullptr);
+    };
+    std::vector<Cand> group;
+    for (auto& c : cands)
+      if (same(cands[0], c)) group.push_back(c);
+    if (group.size() < 2) return;
+    std::map<Name, size_t> elem_loop;  // element variable -> index in group
+    for (size_t g = 0; g < group.size(); ++g) elem_loop[group[g].elem] = g;
+
+    // arrays: every access in the kernel is a[inv + elem] inside a group loop, with one common inv
+    struct Arr { bool ok = true; E inv; ElemSize sz = ElemSize::F32; std::vector<bool> reads, writes; bool seen = false; };
+    std::map<Name, Arr> arrs;
+    for (auto& p : k.params)
+      if (p.ty.is_pointer()) { Arr a; a.reads.assign(group.size(), false); a.writes.assign(group.size(), false); arrs[p.id] = a; }
+    std::set<Name> locals;  // pointer aliases defeat the analysis: any array reachable through one is left alone
+    visit_stmts(k.body, [&](const S& s) {
+      if ((s->k == Stmt::Def && !s->ty.is_scalar()) || (s->k == Stmt::Assign && s->dst->k == Expr::Var && !s->dst->ty.is_scalar()))
+        visit_exprs(s->expr, [&](const E& x) { if (x->k == Expr::Var && arrs.count(x->name)) arrs[x->name].ok = false; });
+    });
+    std::function<void(const E&, int, bool)> scan = [&](const E& e, int g, bool store) {
+      if (!e) return;
+      if ((e->k == Expr::Index || e->k == Expr::AddrOf) && e->args[0]->k == Expr::Var && arrs.count(e->args[0]->name)) {
+        Arr& a = arrs[e->args[0]->name];
+        E inv;
+        bool good = e->k == Expr::Index && g >= 0 && affine_unit(e->args[1], group[g].elem, &inv);
+        if (good) {
+          // inv must be uniform over the block: only the root variable and constants
+          visit_exprs(inv, [&](const E& x) {
+            if (x->k == Expr::Var && x->name != root->id) good = false;
+            if (x->k == Expr::Index || x->k == Expr::ThreadIdx || x->k == Expr::RegElem) good = false;
+          });
+        }
+        if (good && a.seen && (!expr_eq(a.inv, inv) || a.sz != e->ty.sz)) good = false;
+        if (!good) a.ok = false;
+        else {
+          a.seen = true;
+          a.inv = inv;
+          a.sz = e->ty.sz;
+          (store ? a.writes : a.reads)[g] = true;
+        }
+        scan(e->args[1], g, false);
+        return;
+      }
+      if (e->k == Expr::Var && arrs.count(e->name)) { arrs[e->name].ok = false; return; }
+      for (auto& c : e->args) scan(c, g, false);
+    };
+    // accesses under a condition inside a loop body are not cached: a register
+    // slot that was neither loaded nor written must never be stored back
+    std::function<void(const Stmts&, int, bool)> scan_stmts = [&](const Stmts& ss, int g, bool cond) {
+      for (auto& s : ss) {
+        int gg = g;
+        if (g < 0)
+          for (size_t i = 0; i < group.size(); ++i)
+            if (group[i].loop == s) gg = (int)i;
+        int ag = cond ? -1 : gg;  // a conditional access is treated like one outside the loops
+        if (s->dst) scan(s->dst, ag, s->k == Stmt::Assign);
+        if (s->expr) scan(s->expr, ag, false);
+        if (s->lo) scan(s->lo, ag, false);
+        if (s->hi) scan(s->hi, ag, false);
+        for (auto& a : s->args) scan(a, ag, false);
+        bool c = cond || (gg >= 0 && (s->k == Stmt::If || s->k == Stmt::While));
+        scan_stmts(s->body, gg, c);
+        scan_stmts(s->els, gg, c);
+      }
+    };
+    scan_stmts(k.body, -1, false);
+
+    struct Chosen { Name arr, reg; ElemSize sz; E inv; int first, last_write; bool load_first; };
+    std::vector<Chosen> chosen;
+    int64_t slots = group[0].is.slots;
+    for (auto& p : k.params) {
+      auto it = arrs.find(p.id);
+      if (it == arrs.end() || !it->second.ok || !it->second.seen) continue;
+      const Arr& a = it->second;
+      int touched = 0, first = -1, last_write = -1;
+      for (size_t g = 0; g < group.size(); ++g) {
+        if (a.reads[g] || a.writes[g]) { ++touched; if (first < 0) first = (int)g; }
+        if (a.writes[g]) last_write = (int)g;
+      }
+      if (touched < 2) continue;
+      int64_t cost = slots * std::max(1, elem_bytes(a.sz) / 4);
+      if (*budget < cost) continue;
+      *budget -= cost;
+      Chosen c;
+      c.arr = p.id;
+      c.reg = gen.fresh("row_" + p.id.s);
+      c.sz = a.sz;
+      c.inv = a.inv;
+      c.first = first;
+      c.last_write = last_write;
+      c.load_first = a.reads[first];
+      chosen.push_back(c);
+    }
+    if (chosen.empty()) return;
+
+    Type ity = Type::scalar(isz);
+    Stmts nb;
+    for (auto& c : chosen) {
+      auto d = std::make_shared<Stmt>();
+      d->k = Stmt::RegDecl;
+      d->id = c.reg;
+      d->ty = Type::scalar(c.sz);
+      d->iv = slots;
+      nb.push_back(d);
+    }
+    for (size_t pos = 0; pos < root->body.size(); ++pos) {
+      const S& s = root->body[pos];
+      int g = -1;
+      for (size_t i = 0; i < group.size(); ++i)
+        if (group[i].loop == s) g = (int)i;
+      if (g < 0) { nb.push_back(s); continue; }
+      const Cand& c = group[g];
+      auto reg_elem = [&](const Chosen& ch) {
+        auto re = std::make_shared<Expr>();
+        re->k = Expr::RegElem;
+        re->ty = Type::scalar(ch.sz);
+        re->name = ch.reg;
+        re->args = {c.is.slot};
+        return E(re);
+      };
+      auto global_elem = [&](const Chosen& ch) {
+        E idx = fold_expr(mk_binop(BinOp::Add, ch.inv, mk_var(c.elem, ity), ity));
+        return mk_index(mk_var(ch.arr, Type::pointer(ch.sz)), idx, Type::scalar(ch.sz));
+      };
+      auto rw = [&](const E& e) -> E {
+        if (e->k == Expr::Index && e->args[0]->k == Expr::Var)
+          for (auto& ch : chosen)
+            if (ch.arr == e->args[0]->name) return reg_elem(ch);
+        return e;
+      };
+      Stmts body = rewrite_stmts(*c.is.body, rw);
+      Stmts head, tail;
+      for (auto& ch : chosen) {
+        if (g == ch.first && ch.load_first) head.push_back(mk_assign(reg_elem(ch), global_elem(ch)));
+        if (g == ch.last_write) tail.push_back(mk_assign(global_elem(ch), reg_elem(ch)));
+      }
+      Stmts full;
+      size_t start = 0;
+      if (c.is.inner) { full.push_back(body[0]); start = 1; }  // the element definition stays first
+      for (auto& h : head) full.push_back(h);
+      for (size_t i = start; i < body.size(); ++i) full.push_back(body[i]);
+      for (auto& t : tail) full.push_back(t);
+      auto ns = clone(s);
+      ns->unroll = true;
+      if (c.is.inner) {
+        auto ni = clone(c.is.inner);
+        ni->body = full;
+        ns->body = {S(ni)};
+      } else {
+        ns->body = full;
+      }
+      nb.push_back(ns);
+    }
+    auto nr = clone(root);
+    nr->body = nb;
+    k.body = {nr};
+  }
+
+  // ================================================================ read-only parameters
+  // A pointer parameter is read-only when nothing in the kernel stores through
+  // it, directly or through a local alias initialised from it.
+  void mark_read_only() {
+    std::set<Name> written;
+    std::map<Name, std::set<Name>> alias_of;
+    std::function<void(const E&, std::set<Name>&)> bases = [&](const E& e, std::set<Name>& out) {
+      if (!e) return;
+      if (e->k == Expr::Var) {
+        auto it = alias_of.find(e->name);
+        if (it != alias_of.end()) out.insert(it->second.begin(), it->second.end());
+        else out.insert(e->name);
+        return;
+      }
+      if (e->k == Expr::AddrOf || e->k == Expr::Index) { bases(e->args[0], out); return; }
+      if (e->k == Expr::IfExpr) { bases(e->args[1], out); bases(e->args[2], out); }
+    };
+    for (int sweep = 0; sweep < 2; ++sweep) {
+      visit_stmts(k.body, [&](const S& s) {
+        if (s->k == Stmt::Def && (s->ty.is_array() || s->ty.is_pointer())) bases(s->expr, alias_of[s->id]);
+        if (s->k == Stmt::Assign && s->dst->k == Expr::Var && (s->dst->ty.is_array() || s->dst->ty.is_pointer()))
+          bases(s->expr, alias_of[s->dst->name]);
+        if (s->k == Stmt::Assign && s->dst->k == Expr::Index) bases(s->dst->args[0], written);
+      });
+    }
+    for (auto& p : k.params) p.read_only = p.ty.is_pointer() && !written.count(p.id);
+  }
+};
 
 }  // namespace
 
 void hip_optimize(Program& p, const Options& opts, NameGen& gen) {
-  (void)opts;
-  (void)gen;
-  for (auto& k : p.kernels) mark_read_only(k);
+  for (auto& k : p.kernels) {
+    Pass pass(k, opts, gen);
+    if (opts.opt_unswitch) pass.unswitch_aliases();
+    if (opts.opt_lds_rows) pass.lds_rows();
+    if (opts.opt_vectorize) k.body = pass.vectorize(k.body);
+    int64_t budget = pass.reg_budget();
+    if (opts.opt_hoist_invariant) k.body = pass.hoist_invariant(k.body, &budget, false);
+    if (opts.opt_reg_cache) pass.reg_cache(&budget);
+    pass.mark_read_only();
+    k.aligned_params = opts.assume_aligned;
+  }
 }
 
 }  // namespace parpy

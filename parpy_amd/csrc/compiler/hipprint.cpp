@@ -171,6 +171,8 @@ struct DevicePrinter {
 
   // ---------------------------------------------------------------- expressions
   std::string ctype(const Type& t) {
+    if (t.k == Type::Pointer && t.mem == Mem::LDS)
+      return "__attribute__((address_space(3))) " + std::string(elem_ctype(t.sz)) + "*";
     if (t.k == Type::Pointer) return std::string(elem_ctype(t.sz)) + "*";
     if (t.k == Type::Tensor && !t.shape.empty()) return std::string(elem_ctype(t.sz)) + "*";
     if (t.k == Type::Tensor) return elem_ctype(t.sz);
@@ -301,8 +303,14 @@ struct DevicePrinter {
           case UnOp::Sub: return "(-" + a + ")";
           case UnOp::Not: return "(!" + a + ")";
           case UnOp::BitNeg: return "(~" + a + ")";
-          case UnOp::Exp: return call(math_fn("exp", f16 ? ElemSize::F32 : sz, true));
-          case UnOp::Log: return call(math_fn("log", f16 ? ElemSize::F32 : sz, true));
+          // single precision: the hardware base-2 instructions with the scale folded in
+          // (v_exp_f32 / v_log_f32, about 1 ulp, no denormal fix-up)
+          case UnOp::Exp:
+            if (sz == ElemSize::F32) return "__builtin_amdgcn_exp2f(1.44269504088896341f * " + paren(a) + ")";
+            return call(math_fn("exp", f16 ? ElemSize::F32 : sz, true));
+          case UnOp::Log:
+            if (sz == ElemSize::F32) return "(0.693147180559945309f * __builtin_amdgcn_logf" + paren(a) + ")";
+            return call(math_fn("log", f16 ? ElemSize::F32 : sz, true));
           case UnOp::Cos: return call(math_fn("cos", f16 ? ElemSize::F32 : sz, true));
           case UnOp::Sin: return call(math_fn("sin", f16 ? ElemSize::F32 : sz, true));
           case UnOp::Sqrt: return call(math_fn("sqrt", f16 ? ElemSize::F32 : sz, false));
@@ -436,6 +444,15 @@ struct DevicePrinter {
       // every thread runs the same, compile-time known number of iterations
       int64_t per = extent / N;
       std::string k = v + "_k";
+      {
+        // the iteration counter can be named by the memory passes (register array slots)
+        Interval kr;
+        kr.known = true;
+        kr.lo = 0;
+        kr.hi = per - 1;
+        ranges[Name{k, 0}] = kr;
+        narrow_vars.insert(Name{k, 0});
+      }
       if (s->unroll) os << ind(n) << "#pragma unroll\n";
       os << ind(n) << "for (int " << k << " = 0; " << k << " < " << per << "; ++" << k << ") {\n";
       os << ind(n + 2) << vty << " " << v << " = " << init("(" + idx + " + " + k + " * " + std::to_string(N) + ")") << ";\n";
@@ -510,7 +527,8 @@ struct DevicePrinter {
         break;
       }
       case Stmt::LdsDecl:
-        lds_decls.push_back("__shared__ " + std::string(elem_ctype(s->ty.sz)) + " " + s->id.str() + "[" + std::to_string(s->iv) + "];");
+        lds_decls.push_back("__shared__ __attribute__((aligned(16))) " + std::string(elem_ctype(s->ty.sz)) + " " + s->id.str() + "[" +
+                            std::to_string(s->iv) + "];");
         break;
       case Stmt::RegDecl:
         os << ind(n) << elem_ctype(s->ty.sz) << " " << s->id.str() << "[" << s->iv << "];\n";
@@ -546,6 +564,11 @@ struct DevicePrinter {
     }
     out << ") {\n";
     for (auto& d : lds_decls) out << "  " << d << "\n";
+    if (k.aligned_params)
+      for (auto& p : k.params)
+        if (p.ty.k == Type::Pointer)
+          out << "  " << p.id.str() << " = (" << (p.read_only ? "const " : "") << elem_ctype(p.ty.sz) << "*)__builtin_assume_aligned("
+              << p.id.str() << ", 16);\n";
     out << body << "}\n";
     return out.str();
   }

@@ -98,6 +98,7 @@ struct Plan {
   std::vector<HStmt> body;
   std::vector<Val> env;
   int64_t launches = 0;
+  hipEvent_t ev_start = nullptr, ev_stop = nullptr;  // created on the first timed run
 };
 
 struct PlanBuilder {
@@ -554,10 +555,26 @@ int32_t parpy_hip_plan_run(void* plan, void* const* args, int32_t nargs) {
   return run_stmts(p, p.body);
 }
 
+int32_t parpy_hip_plan_run_timed(void* plan, void* const* args, int32_t nargs, float* elapsed_ms) {
+  Plan& p = *(Plan*)plan;
+  if (!p.ev_start) {
+    if (int32_t rc = check(hipEventCreate(&p.ev_start), "hipEventCreate")) return rc;
+    if (int32_t rc = check(hipEventCreate(&p.ev_stop), "hipEventCreate")) return rc;
+  }
+  if (int32_t rc = check(hipEventRecord(p.ev_start, nullptr), "hipEventRecord")) return rc;
+  if (int32_t rc = parpy_hip_plan_run(plan, args, nargs)) return rc;
+  if (int32_t rc = check(hipEventRecord(p.ev_stop, nullptr), "hipEventRecord")) return rc;
+  if (int32_t rc = check(hipEventSynchronize(p.ev_stop), "hipEventSynchronize")) return rc;
+  return check(hipEventElapsedTime(elapsed_ms, p.ev_start, p.ev_stop), "hipEventElapsedTime");
+}
+
 int64_t parpy_hip_plan_launch_count(void* plan) { return ((Plan*)plan)->launches; }
 
 int32_t parpy_hip_plan_destroy(void* plan) {
-  delete (Plan*)plan;
+  Plan* p = (Plan*)plan;
+  if (p->ev_start) (void)hipEventDestroy(p->ev_start);
+  if (p->ev_stop) (void)hipEventDestroy(p->ev_stop);
+  delete p;
   return 0;
 }
 

@@ -213,6 +213,17 @@ class CompileOptions:
         self.includes = []
         self.libs = []
         self.extra_flags = []
+        # HIP memory-codegen switches; None keeps the compiler's default (on).
+        # They exist so that tests and benchmarks can measure what each buys.
+        self.opt_vectorize = None
+        self.opt_lds_rows = None
+        self.opt_reg_cache = None
+        self.opt_hoist_invariant = None
+        self.opt_narrow_index = None
+        self.opt_mfma_sddmm = None
+        self.opt_unswitch = None
+        self.reg_budget = None       # registers per thread the caching passes may claim (None: by block size)
+        self.assume_aligned = None   # set by the driver: False when an array argument is not 16-byte aligned
 
     @property
     def max_thread_blocks_per_cluster(self):

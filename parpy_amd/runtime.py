@@ -67,6 +67,8 @@ def init_library(libpath):
     lib.parpy_hip_plan_create.restype = i32
     lib.parpy_hip_plan_run.argtypes = [vp, ctypes.POINTER(vp), i32]
     lib.parpy_hip_plan_run.restype = i32
+    lib.parpy_hip_plan_run_timed.argtypes = [vp, ctypes.POINTER(vp), i32, ctypes.POINTER(ctypes.c_float)]
+    lib.parpy_hip_plan_run_timed.restype = i32
     lib.parpy_hip_plan_launch_count.argtypes = [vp]
     lib.parpy_hip_plan_launch_count.restype = i64
     lib.parpy_hip_plan_destroy.argtypes = [vp]

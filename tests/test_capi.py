@@ -1,0 +1,56 @@
+"""The two C-ABI libraries load and export every symbol their headers declare (no GPU calls)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared(header):
+    text = open(os.path.join(ROOT, "include", header)).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(parpy_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_runtime_library_exports():
+    from parpy_amd import runtime
+    lib = ctypes.CDLL(str(runtime.PARPY_HIP_BASE_LIB_PATH))
+    names = _declared("parpy_hip.h")
+    assert {"parpy_init", "parpy_sync", "parpy_alloc_buffer", "parpy_memcpy", "parpy_memset", "parpy_free_buffer",
+            "parpy_get_error_message", "parpy_hip_compile", "parpy_hip_plan_run"} <= set(names)
+    for n in names:
+        assert hasattr(lib, n), n
+
+
+def test_compiler_library_exports():
+    from parpy_amd import compiler
+    lib = ctypes.CDLL(str(compiler.LIB_PATH))
+    names = _declared("parpy_hipc.h")
+    assert {"parpy_hipc_parse", "parpy_hipc_compile", "parpy_hipc_fun_print", "parpy_hipc_fun_name"} <= set(names)
+    for n in names:
+        assert hasattr(lib, n), n
+
+
+def test_hiprtc_compile_error_path():
+    """A broken source fails through the C ABI with the compiler log as message (test/test_cuda.py:143-153)."""
+    import parpy_amd as parpy
+    from parpy_amd.compile import hiprtc_compile
+    with pytest.raises(RuntimeError, match="Compilation of generated HIP code failed"):
+        hiprtc_compile("extern \"C\" __global__ void k(float* a) { a[0] = undeclared_name; }", parpy.CompileOptions())
+
+
+def test_plan_rejects_malformed_text_and_wrong_arity():
+    from parpy_amd import runtime
+    lib = runtime.load_hip_runtime_lib()
+    plan = ctypes.c_void_p()
+    assert lib.parpy_hip_plan_create(None, b"(not-a-plan)", ctypes.byref(plan)) != 0
+    assert b"invalid launch plan" in lib.parpy_get_error_message()
+    text = b'(plan "f" (params ("x" ptr)) (kernels) (body ))'
+    assert lib.parpy_hip_plan_create(None, text, ctypes.byref(plan)) == 0
+    args = (ctypes.c_void_p * 2)(None, None)
+    assert lib.parpy_hip_plan_run(plan, args, 2) != 0
+    assert b"expects 1 pointer arguments" in lib.parpy_get_error_message()
+    assert lib.parpy_hip_plan_run(plan, args, 1) != 0   # no module loaded: refuses to run
+    assert lib.parpy_hip_plan_destroy(plan) == 0

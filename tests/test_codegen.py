@@ -1,0 +1,290 @@
+"""Code generation without a GPU: grid mapping, kernel structure, front-end errors.
+
+Follows the reference's codegen-only style (test/test_reduce.py:189-239,
+test/test_forward.py:209-221, test/test_softmax.py:55-65): print_compiled on
+host arrays, regular expressions on the launch lines, and -- stronger than the
+reference, which cannot do it without nvcc -- every generated module is pushed
+through hiprtc for gfx950.
+"""
+import re
+
+import numpy as np
+import pytest
+
+import parpy_amd as parpy
+from parpy_amd import workloads as W
+from parpy_amd.compile import hiprtc_compile
+
+import kernels as K
+
+
+def opts_for(p, **kw):
+    o = parpy.par(p)
+    for k, v in kw.items():
+        setattr(o, k, v)
+    return o
+
+
+def compiles(listing, opts=None):
+    code = hiprtc_compile(listing[:listing.index("// host side")], opts or parpy.CompileOptions())
+    assert len(code) > 0
+    return listing
+
+
+def launch(listing):
+    return re.findall(r"<<<dim3\((\d+), (\d+), (\d+)\), dim3\((\d+), (\d+), (\d+)\)", listing)
+
+
+# ---------------------------------------------------------------- grid mapping (src/gpu/par.rs:105-335 with 64-lane waves)
+@pytest.mark.parametrize("fn", K.ROW_REDUCTIONS)
+def test_reduction_grids(fn):
+    N, M = 100, 50
+    x = np.zeros((N, M), dtype=np.float32)
+    out = np.zeros(N, dtype=np.float32)
+    s1 = compiles(parpy.print_compiled(fn, [x, out, N], opts_for({'outer': parpy.threads(N)})))
+    assert launch(s1) == [("1", "1", "1", "128", "1", "1")]          # 100 threads rounded up to two wavefronts
+    s2 = compiles(parpy.print_compiled(fn, [x, out, N], opts_for({'outer': parpy.threads(N), 'inner': parpy.threads(128)})))
+    assert launch(s2) == [("1", "100", "1", "128", "1", "1")]
+    s3 = compiles(parpy.print_compiled(fn, [x, out, N], opts_for({'outer': parpy.threads(N), 'inner': parpy.threads(1024).tpb(128)})))
+    assert launch(s3)[0] == ("1", "8", "100", "128", "1", "1")       # multi-block: block index becomes an outer level
+    assert launch(s3)[1] == ("1", "100", "1", "64", "1", "1")        # 8 partials reduced by one wavefront
+    assert "parpy_alloc_buffer(3200)" in s3 and "parpy_free_buffer" in s3
+
+
+@pytest.mark.parametrize("fn", K.FULL_REDUCTIONS)
+def test_full_reduction_compiles(fn):
+    x = np.zeros((100, 50), dtype=np.float32)
+    out = np.zeros(100, dtype=np.float32)
+    s = compiles(parpy.print_compiled(fn, [x, out, 100], opts_for({'outer': parpy.threads(128)})))
+    assert launch(s) == [("1", "1", "1", "128", "1", "1")]
+
+
+def test_irregular_thread_count_rounds_to_wavefront():
+    x = np.zeros((100, 83), dtype=np.float32)
+    s = parpy.print_compiled(K.sum_rows, [x, np.zeros(100, dtype=np.float32), 100],
+                             opts_for({'outer': parpy.threads(100), 'inner': parpy.threads(83)}))
+    assert launch(s) == [("1", "100", "1", "128", "1", "1")]
+    assert "parpy_block_reduce<parpy_op_add, 2>" in s
+
+
+def test_single_wave_reduction_uses_no_lds():
+    x = np.zeros((10, 64), dtype=np.float32)
+    s = compiles(parpy.print_compiled(K.max_rows, [x, np.zeros(10, dtype=np.float32), 10],
+                                      opts_for({'outer': parpy.threads(10), 'inner': parpy.threads(64)})))
+    assert "parpy_wave_reduce<parpy_op_max>" in s and "__shared__" not in s.split("extern \"C\" __global__")[1]
+
+
+def test_tpb_must_be_a_multiple_of_the_wavefront():
+    with pytest.raises(RuntimeError, match="divisible by 64"):
+        parpy.threads(128).tpb(96)
+    assert parpy.threads(128).tpb(192)._tpb == 192
+    with pytest.raises(RuntimeError, match="only be set once"):
+        parpy.threads(4).threads(8)
+
+
+def test_thread_blocks_over_threads_dimension():
+    # one parallel level with more threads than a block holds: blocks x threads on X with a guard
+    x = np.zeros(3000, dtype=np.float32)
+    s = compiles(parpy.print_compiled(K.axpy, [2.0, x, x, x.copy(), 3000], opts_for({'N': parpy.threads(3000)})))
+    assert launch(s) == [("3", "1", "1", "1024", "1", "1")]
+    assert re.search(r"< 3000", s)
+
+
+def test_strided_reduction_loop():
+    x = np.zeros((10, 4096), dtype=np.float32)
+    y = np.zeros(10, dtype=np.float32)
+    s = compiles(parpy.print_compiled(K.odd_entries_sum, [x, y, 10, 4096],
+                                      opts_for({'N': parpy.threads(10), 'M': parpy.threads(64).reduce()})))
+    assert launch(s) == [("1", "10", "1", "64", "1", "1")]
+    s = compiles(parpy.print_compiled(K.odd_entries_sum, [x, y, 10, 4096],
+                                      opts_for({'N': parpy.threads(10), 'M': parpy.threads(2048).reduce()})))
+    assert launch(s)[0] == ("1", "2", "10", "1024", "1", "1")
+
+
+# ---------------------------------------------------------------- kernels of the five workloads
+def test_softmax_is_one_kernel_and_row_resident():
+    N, M = 256, 4096
+    x = np.zeros((N, M), dtype=np.float32)
+    s = compiles(parpy.print_compiled(W.softmax, [x, N, M, x.copy()], opts_for({'N': parpy.threads(N), 'M': parpy.threads(1024)})))
+    assert launch(s) == [("1", "256", "1", "1024", "1", "1")]
+    body = s.split("extern \"C\" __global__")[1]
+    # register caching: x is read from memory once and out is written once
+    assert len(re.findall(r"= x_\d+\[", body)) == 1 and len(re.findall(r"\n\s+out_\d+\[.*\] = ", body)) == 1
+    s0 = compiles(parpy.print_compiled(W.softmax, [x, N, M, x.copy()],
+                                       opts_for({'N': parpy.threads(N), 'M': parpy.threads(1024)}, opt_reg_cache=False)))
+    assert len(re.findall(r"x_\d+\[", s0.split("extern \"C\" __global__")[1])) >= 2
+
+
+def _hmm_args(k, n=4, maxlen=30):
+    hmm, seqs = W.synthetic_hmm(k, n_inst=n, min_len=10, max_len=maxlen)
+    S = hmm["num_states"]
+    a = np.zeros((n, S), dtype=np.float32)
+    return hmm, seqs, [hmm, seqs, np.zeros(n, dtype=np.float32), a, a.copy()]
+
+
+def test_hmm_single_block_is_one_kernel_with_lds_rows():
+    hmm, seqs, args = _hmm_args(5)
+    s = compiles(parpy.print_compiled(W.forward_syn, args, opts_for({'inst': parpy.threads(4), 'state': parpy.threads(256)})))
+    assert launch(s) == [("1", "4", "1", "256", "1", "1")]
+    assert len(re.findall(r"__shared__ __attribute__\(\(aligned\(16\)\)\) float lds_alpha", s)) == 2
+    assert "inv_hmm_trans1" in s and "inv_hmm_stay" in s             # transition rows live in registers
+    inner = s[s.index("for (int t_"):]
+    assert not re.search(r"(?<!inv_)hmm_trans1_\d+\[", inner.split("__syncthreads")[0])   # ... and are not re-read every step
+    s0 = compiles(parpy.print_compiled(W.forward_syn, args, opts_for({'inst': parpy.threads(4), 'state': parpy.threads(256)},
+                                                                      opt_lds_rows=False, opt_hoist_invariant=False, opt_vectorize=False)))
+    assert "lds_alpha" not in s0 and "inv_hmm" not in s0
+
+
+def test_hmm_multi_block_hoists_time_loop_to_host():
+    hmm, seqs, args = _hmm_args(5, maxlen=20)
+    s = compiles(parpy.print_compiled(W.forward_syn, args, opts_for({'inst': parpy.threads(4), 'state': parpy.threads(2048).tpb(512)})))
+    host = s[s.index("// host side"):]
+    assert re.search(r"for \(int64_t t_\d+ = 1; t_\d+ < \d+; t_\d+ \+= 1\) \{\n\s+forward_syn_inst_\d+<<<dim3\(4, 4, 1\), dim3\(512, 1, 1\)", host)
+    assert host.count("<<<") >= 5   # init, step, and the split reductions
+
+
+def test_reference_model_kernel_compiles(golden_dir):
+    import os
+    import oracle
+    hmm, seqs = oracle.reference_model_tables(os.path.join(golden_dir, "hmm_3mer_model.npz"), os.path.join(golden_dir, "hmm_signals.npz"))
+    n, S = seqs["num_instances"], hmm["num_states"]
+    a = np.zeros((n, S), dtype=np.float32)
+    for threads in (512, S, 2048):
+        s = compiles(parpy.print_compiled(W.forward_kernel, [hmm, seqs, a, a.copy(), np.zeros(n, dtype=np.float32)],
+                                          opts_for({'inst': parpy.threads(n), 'state': parpy.threads(threads)})))
+        assert len(s) != 0
+
+
+def test_sddmm_kernels_compile():
+    import oracle
+    A, B, crows, cols, vals = W.make_sddmm(128, 16, 0.05)
+    rows = oracle.csr_rows(crows)
+    C = {"rows": rows, "cols": cols, "values": vals, "nnz": len(cols)}
+    s = compiles(parpy.print_compiled(W.sddmm_coo, [A, B, C, np.zeros_like(vals), 1.5, 2.0], opts_for({"nnz": parpy.threads(len(cols))})))
+    assert launch(s) == [("1", "1", "1", "832", "1", "1")] or launch(s)[0][3] in ("832", "1024")
+    s = compiles(parpy.print_compiled(W.sddmm_decompress_csr, [crows, np.zeros_like(cols), 128],
+                                      opts_for({"N": parpy.threads(128), "M": parpy.threads(64)})))
+    assert launch(s) == [("1", "128", "1", "64", "1", "1")]
+
+
+def test_other_shapes_compile():
+    x = np.zeros(64, dtype=np.float32)
+    compiles(parpy.print_compiled(K.saxpy_slices, [2.0, x, x, x.copy()], opts_for({'N': parpy.threads(64)})))
+    d = {"n": 64, "scale": np.float32(2.0), "x": x, "shift": np.zeros(4, dtype=np.float32)}
+    s = compiles(parpy.print_compiled(K.dict_scale, [d, x.copy()], opts_for({'N': parpy.threads(64)})))
+    assert "2.0f" in s                                                # dictionary scalars are folded into the code
+    xi = np.ones(64, dtype=np.int64)
+    compiles(parpy.print_compiled(K.collatz_steps, [xi, np.zeros(64, dtype=np.int32), 64], opts_for({'N': parpy.threads(64)})))
+    s = compiles(parpy.print_compiled(K.gpu_context_fill, [np.zeros(2, dtype=np.float32)], parpy.CompileOptions()))
+    assert launch(s) == [("1", "1", "1", "64", "1", "1")]
+    m = np.zeros((8, 128), dtype=np.float32)
+    compiles(parpy.print_compiled(K.column_sums, [m, np.zeros(128, dtype=np.float32), 8, 128], opts_for({'M': parpy.threads(128)})))
+
+
+def test_generated_code_is_deterministic_and_option_sensitive():
+    x = np.zeros((64, 256), dtype=np.float32)
+    out = np.zeros(64, dtype=np.float32)
+    o = opts_for({'outer': parpy.threads(64), 'inner': parpy.threads(64)})
+    a = parpy.print_compiled(K.sum_rows, [x, out, 64], o)
+    assert a == parpy.print_compiled(K.sum_rows, [x, out, 64], o)
+    assert a != parpy.print_compiled(K.sum_rows, [x, out, 64], opts_for({'outer': parpy.threads(64), 'inner': parpy.threads(128)}))
+    assert "int64_t" in parpy.print_compiled(K.sum_rows, [x, out, 64], opts_for({'outer': parpy.threads(64)}, opt_narrow_index=False)).split("__global__")[1]
+
+
+# ---------------------------------------------------------------- front-end and type errors
+def test_missing_parallelism_is_rejected():
+    x = np.zeros((4, 4), dtype=np.float32)
+    with pytest.raises(RuntimeError, match="does not contain any parallelism"):
+        parpy.print_compiled(K.sum_rows, [x, np.zeros(4, dtype=np.float32), 4], parpy.CompileOptions())
+
+
+def test_opts_keyword_is_required():
+    f = parpy.jit(K.axpy)
+    with pytest.raises(RuntimeError, match="Missing required keyword argument opts"):
+        f(1.0, None, None, None, 4)
+    with pytest.raises(RuntimeError, match="unsupported keyword arguments"):
+        f(1.0, None, None, None, 4, opts=parpy.CompileOptions(), extra=1)
+
+
+def test_unsupported_constructs():
+    def loop_over_list(x, N):
+        parpy.label('N')
+        for i in [1, 2, 3]:
+            x[i] = 0.0
+
+    def chained_compare(x, N):
+        parpy.label('N')
+        for i in range(N):
+            if 0 < i < 3:
+                x[i] = 0.0
+
+    def stepped_slice(x, y):
+        parpy.label('N')
+        y[:] = x[::2]
+
+    def label_on_if(x, N):
+        parpy.label('N')
+        if N > 0:
+            x[0] = 0.0
+
+    with pytest.raises(RuntimeError, match="range builtin"):
+        parpy.jit(loop_over_list)
+    with pytest.raises(RuntimeError, match="Sequences of comparisons"):
+        parpy.jit(chained_compare)
+    with pytest.raises(RuntimeError, match="step size"):
+        parpy.jit(stepped_slice)
+    with pytest.raises(RuntimeError, match="non-parallelizable statement"):
+        parpy.jit(label_on_if)
+
+
+def test_type_errors_carry_the_source_line():
+    def int_plus_float(x, N):
+        parpy.label('N')
+        for i in range(N):
+            x[i] = x[i] + i
+
+    def unknown_name(x, N):
+        parpy.label('N')
+        for i in range(N):
+            x[i] = y_undefined
+
+    x = np.zeros(4, dtype=np.float32)
+    with pytest.raises(TypeError) as e:
+        parpy.print_compiled(int_plus_float, [x, 4], opts_for({'N': parpy.threads(4)}))
+    assert "x[i] = x[i] + i" in str(e.value)
+    with pytest.raises(NameError, match="unknown variable y_undefined"):
+        parpy.jit(unknown_name)
+    with pytest.raises(TypeError, match="out of range"):
+        def oob(x):
+            parpy.label('N')
+            for i in range(4):
+                x[i] = x[7]
+        parpy.print_compiled(oob, [x], opts_for({'N': parpy.threads(4)}))
+
+
+def test_inconsistent_parallel_structure_is_rejected():
+    def two_loops(x, y, N):
+        parpy.label('N')
+        for i in range(N):
+            parpy.label('A')
+            for j in range(64):
+                x[i, j] = 1.0
+            parpy.label('B')
+            for j in range(64):
+                y[i, j] = 2.0
+
+    x = np.zeros((4, 64), dtype=np.float32)
+    with pytest.raises(RuntimeError, match="inconsistent parallel structure"):
+        parpy.print_compiled(two_loops, [x, x.copy(), 4], opts_for({'N': parpy.threads(4), 'A': parpy.threads(64), 'B': parpy.threads(128)}))
+
+
+def test_buffers_reject_strided_and_read_only_arrays():
+    x = np.zeros((8, 8), dtype=np.float32)
+    with pytest.raises((RuntimeError, ValueError)):
+        parpy.print_compiled(K.sum_rows, [x[:, ::2], np.zeros(8, dtype=np.float32), 8], opts_for({'outer': parpy.threads(8)}))
+    ro = np.zeros(8, dtype=np.float32)
+    ro.setflags(write=False)
+    with pytest.raises((RuntimeError, ValueError)):
+        parpy.print_compiled(K.axpy, [1.0, ro, ro, ro, 8], opts_for({'N': parpy.threads(8)}))
+    with pytest.raises(RuntimeError, match="nested dictionary"):
+        parpy.print_compiled(K.dict_scale, [{"n": {"a": 1}}, x], opts_for({'N': parpy.threads(8)}))

@@ -1,0 +1,314 @@
+"""GPU parity tests: compiled kernels against the CPU oracle and the reference's golden vectors.
+
+Everything here runs through the C ABI of the runtime library
+(parpy_hip_plan_run) on a real MI355X.  Tolerances are the reference's own:
+reductions atol 1e-4 (test/test_reduce.py:81-85), softmax atol 1e-5
+(test/test_softmax.py:35-40), HMM forward atol = rtol = 1e-5
+(test/test_forward.py:176-178), SDDMM atol = rtol = 1e-5 (benchmarks/sddmm.py:86-103).
+"""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import parpy_amd as parpy
+from parpy_amd import workloads as W
+
+import kernels as K
+
+pytestmark = pytest.mark.gpu
+
+HIP = parpy.CompileBackend.Hip
+
+
+def opts_for(p, **kw):
+    o = parpy.par(p)
+    o.backend = HIP
+    for k, v in kw.items():
+        setattr(o, k, v)
+    return o
+
+
+def np_reduce(fn, x):
+    op = fn.__name__.split("_")[0]
+    f = {"sum": np.sum, "prod": np.prod, "max": np.max, "min": np.min}[op]
+    if fn in K.FULL_REDUCTIONS:
+        out = np.zeros(x.shape[0], dtype=x.dtype)
+        out[0] = f(x.astype(np.float64))
+        return out
+    return f(x.astype(np.float64), axis=1).astype(x.dtype)
+
+
+REDUCE_CASES = [
+    ("outer", 100, 50, lambda N, M: {'outer': parpy.threads(N)}),
+    ("outer+inner", 100, 50, lambda N, M: {'outer': parpy.threads(N), 'inner': parpy.threads(128)}),
+    ("irregular", 100, 83, lambda N, M: {'outer': parpy.threads(N), 'inner': parpy.threads(M)}),
+    ("multi-block", 100, 2048, lambda N, M: {'outer': parpy.threads(N), 'inner': parpy.threads(M).tpb(512)}),
+]
+
+
+@pytest.mark.parametrize("fn", K.ROW_REDUCTIONS + K.FULL_REDUCTIONS, ids=lambda f: f.__name__)
+@pytest.mark.parametrize("case", REDUCE_CASES, ids=lambda c: c[0])
+def test_reductions(fn, case):
+    _, N, M, spec = case
+    rng = np.random.default_rng(1234)
+    # products over 2048 normal values under- or overflow; keep them near one
+    x = rng.standard_normal((N, M)).astype(np.float32)
+    if fn.__name__.startswith("prod"):
+        x = (1.0 + 0.001 * x).astype(np.float32)
+    p = spec(N, M)
+    if fn in K.FULL_REDUCTIONS:
+        p = {'outer': p.get('inner', p['outer'])} if case[0] != "outer" else p
+        if case[0] == "multi-block":
+            p = {'outer': parpy.threads(2048).tpb(512)}
+    out = np.zeros(N, dtype=np.float32)
+    parpy.jit(fn)(x, out, N, opts=opts_for(p))
+    want = np_reduce(fn, x)
+    tol = 1e-4 if not fn.__name__.startswith("sum_2d") else 2e-3
+    assert np.allclose(out, want, atol=tol, rtol=1e-5), (np.abs(out - want).max(), fn.__name__, case[0])
+
+
+@pytest.mark.parametrize("threads", [64, 2048])
+def test_strided_reduction(threads):
+    N, M = 10, 4096
+    x = np.random.default_rng(1).standard_normal((N, M)).astype(np.float32)
+    out = np.zeros(N, dtype=np.float32)
+    parpy.jit(K.odd_entries_sum)(x, out, N, M, opts=opts_for({'N': parpy.threads(N), 'M': parpy.threads(threads).reduce()}))
+    assert np.allclose(out, x[:, 1::2].astype(np.float64).sum(1), atol=1e-4)
+
+
+def test_rowsum_full_size():
+    N, M = 1024, 65536
+    x = W.make_rowsum(N, M)
+    xd = torch.from_numpy(x).cuda()
+    want = oracle.row_reduce(x).astype(np.float32)
+    for threads in (256, 1024):
+        out = torch.zeros(N, dtype=torch.float32, device="cuda")
+        W.sum_rows(xd, out, N, opts=opts_for({'outer': parpy.threads(N), 'inner': parpy.threads(threads)}))
+        assert np.allclose(out.cpu().numpy(), want, atol=1e-4, rtol=1e-5)
+
+
+@pytest.mark.parametrize("p", [{"N": 256}, {"N": 256, "M": 128}, {"N": 256, "M": 512}])
+def test_softmax_small(p):
+    N, M = 256, 512
+    x = W.make_softmax(N, M)
+    out = torch.zeros_like(x)
+    W.softmax(x, N, M, out, opts=opts_for({k: parpy.threads(v) for k, v in p.items()}))   # host tensors: copied in and back
+    assert torch.allclose(out, torch.softmax(x, 1), atol=1e-5)
+
+
+def test_softmax_full_size_and_without_register_caching():
+    N, M = 16384, 4096
+    x = W.make_softmax(N, M)
+    xd = x.cuda()
+    want = torch.softmax(x, 1)
+    for kw in ({}, {"opt_reg_cache": False, "opt_vectorize": False}):
+        out = torch.zeros_like(xd)
+        W.softmax(xd, N, M, out, opts=opts_for({'N': parpy.threads(N), 'M': parpy.threads(1024)}, **kw))
+        got = out.cpu()
+        assert torch.allclose(got, want, atol=1e-5, rtol=1e-5)
+        assert torch.allclose(got.sum(1), torch.ones(N), atol=1e-5)
+
+
+# ---------------------------------------------------------------- HMM forward
+def _golden(golden_dir, k):
+    hmm, seqs = oracle.reference_model_tables(os.path.join(golden_dir, f"hmm_{k}mer_model.npz"),
+                                              os.path.join(golden_dir, "hmm_signals.npz"))
+    exp = np.loadtxt(os.path.join(golden_dir, f"hmm_{k}mer_expected.txt"), dtype=np.float32)
+    return hmm, seqs, exp
+
+
+def _run_reference_model(hmm, seqs, threads, **kw):
+    hd, sd = W.to_device(hmm), W.to_device(seqs)
+    n, S = seqs["num_instances"], hmm["num_states"]
+    a1 = torch.zeros((n, S), dtype=torch.float32, device="cuda")
+    a2 = torch.zeros_like(a1)
+    res = torch.zeros(n, dtype=torch.float32, device="cuda")
+    W.forward_kernel(hd, sd, a1, a2, res, opts=opts_for({'inst': parpy.threads(n), 'state': parpy.threads(threads)}, **kw))
+    return res.cpu().numpy()
+
+
+@pytest.mark.parametrize("threads", [512, 1024, 2048])
+def test_forward_3mer_golden(golden_dir, threads):
+    """test_forward_single_block / test_forward_multi_block of the reference (test/test_forward.py:182-207)."""
+    hmm, seqs, exp = _golden(golden_dir, 3)
+    got = _run_reference_model(hmm, seqs, threads)
+    assert np.allclose(got, exp, atol=1e-5, rtol=1e-5), np.abs(got - exp).max()
+
+
+def test_forward_3mer_golden_unoptimised(golden_dir):
+    hmm, seqs, exp = _golden(golden_dir, 3)
+    got = _run_reference_model(hmm, seqs, 512, opt_lds_rows=False, opt_vectorize=False, opt_hoist_invariant=False,
+                               opt_narrow_index=False)
+    assert np.allclose(got, exp, atol=1e-5, rtol=1e-5), np.abs(got - exp).max()
+
+
+def test_forward_5mer_golden(golden_dir):
+    """The reference's benchmark validation (benchmarks/forward.py:481-482,518): 16384 states, 100 reads."""
+    hmm, seqs, exp = _golden(golden_dir, 5)
+    got = _run_reference_model(hmm, seqs, 1024)
+    assert np.allclose(got, exp, atol=1e-5, rtol=1e-5), np.abs(got - exp).max()
+
+
+def _run_synthetic(hmm, seqs, threads, **kw):
+    hd, sd = W.to_device(hmm), W.to_device(seqs)
+    n, S = seqs["num_instances"], hmm["num_states"]
+    a1 = torch.zeros((n, S), dtype=torch.float32, device="cuda")
+    a2 = torch.zeros_like(a1)
+    res = torch.zeros(n, dtype=torch.float32, device="cuda")
+    W.forward_syn(hd, sd, res, a1, a2, opts=opts_for({'inst': parpy.threads(n), 'state': parpy.threads(threads)}, **kw))
+    return res.cpu().numpy(), a1.cpu().numpy(), a2.cpu().numpy()
+
+
+@pytest.mark.parametrize("k,threads", [(3, 64), (4, 64), (4, 256), (5, 256), (5, 1024), (5, 4096)])
+def test_forward_synthetic_vs_oracle(k, threads):
+    hmm, seqs = W.synthetic_hmm(k, n_inst=16, min_len=1, max_len=300)
+    seqs["lens"][0] = 1   # a read with a single sample: no forward step at all
+    got, a1, a2 = _run_synthetic(hmm, seqs, threads)
+    want, alpha = oracle.hmm_syn_forward(hmm, seqs, np.float32, return_alpha=True)
+    assert np.allclose(got, want, atol=1e-5, rtol=1e-5), np.abs(got - want).max()
+    # the final state vector of every read (which buffer holds it depends on the parity of its length)
+    for i, n in enumerate(seqs["lens"]):
+        final = a1[i] if n % 2 == 1 else a2[i]
+        assert np.allclose(final, alpha[i], atol=2e-3, rtol=1e-5)
+
+
+@pytest.mark.parametrize("flags", [
+    {"opt_lds_rows": False}, {"opt_vectorize": False}, {"opt_hoist_invariant": False}, {"opt_narrow_index": False},
+    {"opt_unswitch": True}, {"opt_lds_rows": False, "opt_vectorize": False, "opt_hoist_invariant": False},
+], ids=lambda f: ",".join(f"{k}={int(v)}" for k, v in f.items()))
+def test_forward_synthetic_each_memory_pass_preserves_results(flags):
+    hmm, seqs = W.synthetic_hmm(5, n_inst=8, min_len=50, max_len=200)
+    base, _, _ = _run_synthetic(hmm, seqs, 256)
+    got, _, _ = _run_synthetic(hmm, seqs, 256, **flags)
+    want = oracle.hmm_syn_forward(hmm, seqs, np.float32)
+    assert np.allclose(got, want, atol=1e-5, rtol=1e-5)
+    assert np.allclose(got, base, atol=1e-3, rtol=0)
+
+
+def test_forward_7mer_full_size_properties():
+    """Full headline shape (16384 states, 100 reads of 5000..15000 samples)."""
+    hmm, seqs = W.synthetic_hmm(7)
+    got, _, _ = _run_synthetic(hmm, seqs, 1024)
+    assert np.all(np.isfinite(got)) and np.all(got < 0)
+    # parity on the four shortest reads against the fp32 oracle at full length
+    sub = np.argsort(seqs["lens"])[:4]
+    want = oracle.hmm_syn_forward(hmm, seqs, np.float32, subset=sub)
+    assert np.allclose(got[sub], want, atol=1e-5, rtol=1e-5), np.abs(got[sub] - want).max()
+    # constant emissions: the log-likelihood is len * c whatever the transitions are
+    c = np.float32(np.log(1.0 / 101.0))
+    hmm_c, seqs_c = W.synthetic_hmm(7, emissions=c)
+    got_c, _, _ = _run_synthetic(hmm_c, seqs_c, 1024)
+    # exact in real arithmetic; fp32 accumulates up to ~1e-4 relative drift over 15000 steps
+    # (the fp32 CPU restatement drifts the same way against fp64, see tests/test_oracle.py)
+    assert np.allclose(got_c, seqs_c["lens"] * float(c), rtol=1e-4, atol=0)
+
+
+def test_forward_all_states_unreachable_gives_neg_inf():
+    hmm, seqs = W.synthetic_hmm(4, n_inst=4, min_len=5, max_len=20)
+    hmm["initial_prob"][:] = -np.inf
+    got, a1, a2 = _run_synthetic(hmm, seqs, 256)
+    assert np.all(np.isnan(got) | np.isneginf(got))          # max = -inf, log(sum(exp(nan))) like the CPU restatement
+    assert np.all(np.isneginf(a1[seqs["lens"] > 1]) | np.isneginf(a2[seqs["lens"] > 1]))
+
+
+# ---------------------------------------------------------------- SDDMM
+@pytest.mark.parametrize("n,k,density", [(256, 32, 0.05), (8192, 128, 0.01)])
+def test_sddmm(n, k, density):
+    A, B, crows, cols, vals = W.make_sddmm(n, k, density)
+    nnz = len(cols)
+    Ad, Bd = torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda()
+    crows_d = torch.from_numpy(crows).cuda()
+    rows_d = torch.zeros(nnz, dtype=torch.int64, device="cuda")
+    W.sddmm_decompress_csr(crows_d, rows_d, n, opts=opts_for({"N": parpy.threads(n), "M": parpy.threads(64)}))
+    rows = oracle.csr_rows(crows)
+    assert np.array_equal(rows_d.cpu().numpy(), rows)          # index work: bit-exact
+    C = {"rows": rows_d, "cols": torch.from_numpy(cols).cuda(), "values": torch.from_numpy(vals).cuda(), "nnz": nnz}
+    D = torch.zeros(nnz, dtype=torch.float32, device="cuda")
+    W.sddmm_coo(Ad, Bd, C, D, 1.5, 2.0, opts=opts_for({"nnz": parpy.threads(nnz).tpb(256)}))
+    want = oracle.sddmm(A, B, rows, cols, vals, alpha=1.5, beta=2.0)
+    got = D.cpu().numpy()
+    bad = np.abs(got - want) > 1e-5 + 1e-5 * np.abs(want)
+    # the reference's own criterion (benchmarks/sddmm.py:93-103): fatal from 5 elements and 5 %
+    assert bad.sum() < 5 or bad.mean() < 0.05, (bad.sum(), np.abs(got - want).max())
+    assert np.abs(got - want).max() < 5e-4
+
+
+# ---------------------------------------------------------------- surface behaviour
+def test_host_arrays_are_copied_back_and_device_arrays_are_shared():
+    N = 1000
+    rng = np.random.default_rng(0)
+    x, y = rng.standard_normal(N).astype(np.float32), rng.standard_normal(N).astype(np.float32)
+    out = np.zeros(N, dtype=np.float32)
+    parpy.jit(K.axpy)(2.5, x, y, out, N, opts=opts_for({'N': parpy.threads(N)}))
+    assert np.allclose(out, 2.5 * x + y, atol=1e-6)
+    xd, yd, od = (torch.from_numpy(a).cuda() for a in (x, y, np.zeros(N, dtype=np.float32)))
+    parpy.jit(K.saxpy_slices)(2.5, xd, yd, od, opts=opts_for({'N': parpy.threads(N)}))
+    parpy.sync(HIP)
+    assert np.allclose(od.cpu().numpy(), 2.5 * x + y, atol=1e-6)
+
+
+def test_dict_arguments_and_scalar_specialisation():
+    x = np.arange(64, dtype=np.float32)
+    shift = np.array([1, 2, 3, 4], dtype=np.float32)
+    f = parpy.jit(K.dict_scale)
+    for scale in (2.0, -3.0):                                     # a new scalar value compiles a new kernel
+        out = np.zeros(64, dtype=np.float32)
+        f({"n": 64, "scale": np.float32(scale), "x": x, "shift": shift}, out, opts=opts_for({'N': parpy.threads(64)}))
+        assert np.allclose(out, scale * x + shift[np.arange(64) % 4])
+
+
+def test_integer_work_is_bit_exact():
+    x = np.array([1, 2, 3, 6, 7, 27, 97, 871] * 8, dtype=np.int64)
+    out = np.zeros(64, dtype=np.int32)
+    parpy.jit(K.collatz_steps)(x, out, 64, opts=opts_for({'N': parpy.threads(64)}))
+
+    def steps(v):
+        n = 0
+        while v != 1:
+            v = v // 2 if v % 2 == 0 else 3 * v + 1
+            n += 1
+        return n
+    assert np.array_equal(out, np.array([steps(int(v)) for v in x], dtype=np.int32))
+
+
+def test_gpu_context_and_sequential_kernel():
+    out = np.zeros(2, dtype=np.float32)
+    parpy.jit(K.gpu_context_fill)(out, opts=opts_for({}))
+    assert out.tolist() == [7.0, 8.0]
+    m = np.random.default_rng(2).standard_normal((8, 128)).astype(np.float32)
+    cs = np.zeros(128, dtype=np.float32)
+    parpy.jit(K.column_sums)(m, cs, 8, 128, opts=opts_for({'M': parpy.threads(128)}))
+    assert np.allclose(cs, m.sum(0), atol=1e-5)
+
+
+def test_compile_string_and_runtime_error_paths():
+    src = 'extern "C" __global__ void twice(float* x, long long n) { long long i = blockIdx.x * 64 + threadIdx.x; if (i < n) x[i] *= 2.0f; }'
+    o = parpy.CompileOptions()
+    o.backend = HIP
+    f = parpy.compile_string("twice", src, o, grid=(2, 1, 1), block=(64, 1, 1))
+    x = torch.arange(100, dtype=torch.float32, device="cuda")
+    f(x, 100)
+    parpy.sync(HIP)
+    assert torch.equal(x.cpu(), torch.arange(100, dtype=torch.float32) * 2)
+    with pytest.raises(RuntimeError, match="Compilation of generated HIP code failed"):
+        parpy.compile_string("broken", "extern \"C\" __global__ void broken() { this is not C++; }", o)
+    g = parpy.compile_string("missing_kernel", src, o)
+    with pytest.raises(RuntimeError):
+        g(x, 100)                                                  # unknown kernel name: module lookup failure
+    from parpy_amd.runtime import _compile_runtime_lib
+    lib = _compile_runtime_lib(HIP)
+    assert not lib.parpy_alloc_buffer(1 << 60)                      # absurd allocation: NULL and a message
+    assert len(lib.parpy_get_error_message()) > 0
+
+
+def test_timed_call_and_launch_count():
+    hmm, seqs = W.synthetic_hmm(4, n_inst=4, min_len=20, max_len=40)
+    hd, sd = W.to_device(hmm), W.to_device(seqs)
+    n, S = 4, 256
+    a1 = torch.zeros((n, S), dtype=torch.float32, device="cuda")
+    res = torch.zeros(n, dtype=torch.float32, device="cuda")
+    ms = parpy.time_call(W.forward_syn, hd, sd, res, a1, torch.zeros_like(a1), opts=opts_for({'inst': parpy.threads(n), 'state': parpy.threads(256)}))
+    assert 0 < ms < 1000
