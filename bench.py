@@ -171,6 +171,38 @@ def bench_sddmm(args, torch, parpy, W):
             "cpu_baseline": cpu}
 
 
+def bench_copy(args, torch, parpy, W):
+    """Plain device copy of 256 MiB compiled from `out[:] = x[:]`: the calibration kernel for the HBM counters."""
+    import numpy as np
+    n = 64 * 1024 * 1024
+    x = torch.arange(n, dtype=torch.float32, device="cuda")
+    out = torch.zeros_like(x)
+    opts = parpy.par({"N": parpy.threads(n // 16).tpb(256)})
+    fn = lambda: W.copy_1d(x, out, opts=opts)
+    timed = lambda: parpy.time_call(W.copy_1d, x, out, opts=opts)
+    wall, dev = _events_ms(fn, timed, args.steps, args.warmup, torch)
+    assert torch.equal(x, out)
+    alg = 2 * n * 4
+    kernel_ms = float(np.median(dev))
+    return {"metric": "device copy 256 MiB ms + achieved HBM GB/s", "value": wall, "unit": "ms/batch", "ms_per_step": wall,
+            "higher_is_better": False, "dtype": "f32", "config": {"workload": "copy_256MiB"},
+            "roofline": {"bound": "hbm", "achieved": alg / (kernel_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": alg / (kernel_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None, "kernel_ms": kernel_ms,
+                         "algorithmic_bytes": alg},
+            "cpu_baseline": None}
+
+
+def _profiled_traffic(name):
+    """HBM bytes per launch from the committed rocprofv3 counter summary of this kernel, or None."""
+    import re
+    path = os.path.join(ROOT, "profiles", f"{name}_kernel.md")
+    try:
+        m = re.search(r"^traffic_bytes_per_launch:\s*(\d+)", open(path).read(), re.M)
+        return int(m.group(1)) if m else None
+    except OSError:
+        return None
+
+
 def _apply_opt_flags(opts, args):
     for name in ("opt_vectorize", "opt_lds_rows", "opt_reg_cache", "opt_hoist_invariant", "opt_narrow_index", "opt_unswitch"):
         v = getattr(args, name)
@@ -185,7 +217,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=2)
-    ap.add_argument("--workload", default="hmm7", choices=["hmm7", "hmm5", "rowsum", "softmax", "sddmm"])
+    ap.add_argument("--workload", default="hmm7", choices=["hmm7", "hmm5", "rowsum", "softmax", "sddmm", "copy"])
     ap.add_argument("--state-threads", type=int, default=1024)
     ap.add_argument("--inner-threads", type=int, default=1024)
     ap.add_argument("--tpb", type=int, default=256)
@@ -215,8 +247,14 @@ def main():
         r = bench_rowsum(args, torch, parpy, W)
     elif args.workload == "softmax":
         r = bench_softmax(args, torch, parpy, W)
+    elif args.workload == "copy":
+        r = bench_copy(args, torch, parpy, W)
     else:
         r = bench_sddmm(args, torch, parpy, W)
+    default_cfg = not any(getattr(args, n) is not None for n in ("opt_vectorize", "opt_lds_rows", "opt_reg_cache",
+                                                                 "opt_hoist_invariant", "opt_narrow_index", "opt_unswitch"))
+    if default_cfg and not args.reg_budget:
+        r["roofline"]["traffic"] = _profiled_traffic(args.workload)
     r.update({"n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "scaling": "weak", "vs_baseline": None,
               "data": "synthetic"})
     print(json.dumps(r))

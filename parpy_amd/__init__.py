@@ -82,10 +82,25 @@ def _check_kwargs(kwargs, fun_name):
     return opts
 
 
+def _all_arrays_aligned(args, nbytes=16):
+    from .buffer import Buffer
+    for a in args:
+        for v in (a.values() if isinstance(a, dict) else [a]):
+            if isinstance(v, Buffer) and len(v.shape) > 0 and v._get_ptr() % nbytes != 0:
+                return False
+    return True
+
+
 def _compile_function(ir_ast, args, opts):
     from .compile import build_code_object, get_wrapper
     from .key import _generate_fast_cache_key, _generate_function_key
+    import copy
     name = compiler.get_function_name(ir_ast)
+    # vector accesses assume 16-byte aligned arrays: true for whole torch allocations,
+    # not for offset views -- those get a specialisation without the assumption
+    if opts.assume_aligned is None and not _all_arrays_aligned(args):
+        opts = copy.copy(opts)
+        opts.assume_aligned = False
     fast_cache_key = _generate_fast_cache_key(ir_ast, args, opts)
     if fast_cache_key in _fun_cache:
         return _fun_cache[fast_cache_key]

@@ -39,6 +39,13 @@ def softmax(x, N, M, out):
         out[i, :] = out[i, :] / s
 
 
+@parpy.jit
+def copy_1d(x, out):
+    """out[:] = x[:] -- a plain streaming copy (counter calibration and bandwidth reference)."""
+    parpy.label('N')
+    out[:] = x[:]
+
+
 # ---------------------------------------------------------------- SDDMM
 @parpy.jit
 def sddmm_decompress_csr(C_crows, C_rows, N):

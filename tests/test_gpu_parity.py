@@ -201,9 +201,9 @@ def test_forward_7mer_full_size_properties():
     c = np.float32(np.log(1.0 / 101.0))
     hmm_c, seqs_c = W.synthetic_hmm(7, emissions=c)
     got_c, _, _ = _run_synthetic(hmm_c, seqs_c, 1024)
-    # exact in real arithmetic; fp32 accumulates up to ~1e-4 relative drift over 15000 steps
-    # (the fp32 CPU restatement drifts the same way against fp64, see tests/test_oracle.py)
-    assert np.allclose(got_c, seqs_c["lens"] * float(c), rtol=1e-4, atol=0)
+    # exact in real arithmetic; adding c = -4.6 to sums of magnitude up to 7e4 (fp32 ulp 0.008) 15000 times
+    # drifts by up to ~2e-4 relative (the fp32 CPU restatement drifts the same way against fp64)
+    assert np.allclose(got_c, seqs_c["lens"] * float(c), rtol=5e-4, atol=0)
 
 
 def test_forward_all_states_unreachable_gives_neg_inf():
@@ -312,3 +312,13 @@ def test_timed_call_and_launch_count():
     res = torch.zeros(n, dtype=torch.float32, device="cuda")
     ms = parpy.time_call(W.forward_syn, hd, sd, res, a1, torch.zeros_like(a1), opts=opts_for({'inst': parpy.threads(n), 'state': parpy.threads(256)}))
     assert 0 < ms < 1000
+
+
+def test_unaligned_views_get_their_own_specialisation():
+    N = 4096
+    base = torch.arange(N + 1, dtype=torch.float32, device="cuda")
+    x = base[1:]                                   # contiguous but only 4-byte aligned
+    out = torch.zeros(N, dtype=torch.float32, device="cuda")
+    W.copy_1d(x, out, opts=opts_for({'N': parpy.threads(N // 4)}))
+    parpy.sync(HIP)
+    assert torch.equal(out, x)
