@@ -362,7 +362,9 @@ struct Options {  // src/option.rs:14-108
   bool opt_narrow_index = true;
   bool opt_mfma_sddmm = true;
   bool opt_unswitch = false;   // measured slower on the HMM kernels (higher register pressure): opt-in
-  int64_t reg_budget = 0;      // 32-bit registers per thread the caching passes may claim (0 = by block size)
+  bool opt_gather_transpose = true;
+  bool opt_nontemporal = true;   // non-temporal stores to arrays a kernel only writes
+  int64_t reg_budget = 0;     // 32-bit registers per thread the caching passes may claim (0 = by block size)
   bool assume_aligned = true;  // array arguments are at least 16-byte aligned
   ElemSize int_size() const { return has_force_int ? force_int : ElemSize::I64; }
   ElemSize float_size() const { return has_force_float ? force_float : ElemSize::F64; }

@@ -945,6 +945,52 @@ struct Pass {
     k.body = {nr};
   }
 
+  // ================================================================ streaming loads
+  // A read-only array that the kernel reads at exactly one place, outside any
+  // sequential loop, is read once per element: its loads are marked
+  // non-temporal (Expr::bv on the Index node) so they do not displace data that
+  // is reused.  Measured on a plain copy: 6.3 instead of 5.8 TB/s.
+  void mark_streaming_loads() {
+    std::map<Name, int> sites;
+    std::set<Name> bad;
+    std::function<void(const E&, bool, bool)> scan = [&](const E& e, bool in_seq, bool is_dst) {
+      if (!e) return;
+      if (e->k == Expr::Index && e->args[0]->k == Expr::Var) {
+        const Name& b = e->args[0]->name;
+        if (is_dst || in_seq || elem_bytes(e->ty.sz) < 4) bad.insert(b);
+        else sites[b]++;
+        scan(e->args[1], in_seq, false);
+        return;
+      }
+      if (e->k == Expr::Var && !e->ty.is_scalar()) { bad.insert(e->name); return; }
+      for (auto& a : e->args) scan(a, in_seq, false);
+    };
+    std::function<void(const Stmts&, bool)> walk = [&](const Stmts& ss, bool in_seq) {
+      for (auto& s : ss) {
+        scan(s->dst, in_seq, s->k == Stmt::Assign);
+        scan(s->expr, in_seq, false);
+        scan(s->lo, in_seq, false);
+        scan(s->hi, in_seq, false);
+        bool seq = in_seq || (s->k == Stmt::For && s->map.k == GpuMap::None && !s->unroll) || s->k == Stmt::While;
+        walk(s->body, seq);
+        walk(s->els, seq);
+      }
+    };
+    walk(k.body, false);
+    std::set<Name> stream;
+    for (auto& p : k.params)
+      if (p.ty.is_pointer() && p.read_only && !bad.count(p.id) && sites[p.id] == 1) stream.insert(p.id);
+    if (stream.empty()) return;
+    k.body = rewrite_stmts(k.body, [&](const E& e) -> E {
+      if (e->k == Expr::Index && e->args[0]->k == Expr::Var && stream.count(e->args[0]->name)) {
+        auto n = std::make_shared<Expr>(*e);
+        n->bv = true;
+        return n;
+      }
+      return e;
+    });
+  }
+
   // ================================================================ read-only parameters
   // A pointer parameter is read-only when nothing in the kernel stores through
   // it, directly or through a local alias initialised from it.
@@ -974,9 +1020,184 @@ struct Pass {
   }
 };
 
+// ================================================================ transposed staging of column gathers
+// A read-only matrix X[K, N] that a kernel only reads as X[d, c] with d the
+// variable of an innermost sequential loop over all K rows and c fixed per
+// thread is a column gather: every step of the loop touches one 4-byte word
+// in each of up to 64 different cache lines per wavefront.  Staging X^T once
+// in a device temporary turns each thread's column into K contiguous words
+// (dwordx4 loads, whole cache lines used).  The transposition costs two
+// passes over X; it is applied to kernels launched once per call.
+struct GatherTranspose {
+  Program& p;
+  const Options& opts;
+  NameGen& gen;
+  ElemSize isz;
+
+  GatherTranspose(Program& prog, const Options& o, NameGen& g) : p(prog), opts(o), gen(g), isz(o.int_size()) {}
+
+  struct Cand { Name arr; int64_t K = 0, N = 0; ElemSize sz = ElemSize::F32; bool ok = true; bool seen = false; };
+
+  void scan_expr(const E& e, const std::vector<std::pair<Name, int64_t>>& seq_loops, std::map<Name, Cand>& cands) {
+    if (!e) return;
+    if ((e->k == Expr::Index || e->k == Expr::AddrOf) && e->args[0]->k == Expr::Var && cands.count(e->args[0]->name)) {
+      Cand& c = cands[e->args[0]->name];
+      bool good = e->k == Expr::Index && e->dim_idx.size() == 2 && e->dim_idx[0]->k == Expr::Var && !seq_loops.empty() &&
+                  e->dim_idx[0]->name == seq_loops.back().first && e->dim_shape[0] == seq_loops.back().second &&
+                  !mentions(e->dim_idx[1], seq_loops.back().first) && !has_load(e->dim_idx[1]);
+      if (good && c.seen && (c.K != e->dim_shape[0] || c.N != e->dim_shape[1])) good = false;
+      if (!good) c.ok = false;
+      else { c.seen = true; c.K = e->dim_shape[0]; c.N = e->dim_shape[1]; c.sz = e->ty.sz; }
+      scan_expr(e->args[1], seq_loops, cands);
+      return;
+    }
+    if (e->k == Expr::Var && cands.count(e->name)) { cands[e->name].ok = false; return; }
+    for (auto& a : e->args) scan_expr(a, seq_loops, cands);
+  }
+
+  void scan(const Stmts& ss, std::vector<std::pair<Name, int64_t>>& seq_loops, std::map<Name, Cand>& cands) {
+    for (auto& s : ss) {
+      scan_expr(s->dst, seq_loops, cands);
+      scan_expr(s->expr, seq_loops, cands);
+      scan_expr(s->lo, seq_loops, cands);
+      scan_expr(s->hi, seq_loops, cands);
+      for (auto& a : s->args) scan_expr(a, seq_loops, cands);
+      bool seq = s->k == Stmt::For && s->map.k == GpuMap::None && s->step == 1 && s->lo->k == Expr::Int && s->lo->iv == 0 &&
+                 s->hi->k == Expr::Int;
+      // only innermost loops qualify: a nested loop hides the enclosing one
+      if (seq) seq_loops.emplace_back(s->id, s->hi->iv);
+      else if (s->k == Stmt::For || s->k == Stmt::While) seq_loops.emplace_back(Name{"", -1}, -1);
+      scan(s->body, seq_loops, cands);
+      if (s->k == Stmt::For || s->k == Stmt::While) seq_loops.pop_back();
+      scan(s->els, seq_loops, cands);
+    }
+  }
+
+  Kernel make_transpose(const Name& x, const Name& xt, const Cand& c) {
+    // one thread per column c; reads are coalesced across the wavefront, each thread writes its own row of X^T
+    Type ity = Type::scalar(isz);
+    Type elem = Type::scalar(c.sz);
+    Name cv = gen.fresh("c"), dv = gen.fresh("d");
+    E ce = mk_var(cv, ity), de = mk_var(dv, ity);
+    E src = mk_index(mk_var(x, Type::pointer(c.sz)), fold_expr(mk_binop(BinOp::Add, mk_binop(BinOp::Mul, de, mk_int(c.N, isz), ity), ce, ity)), elem);
+    E dst = mk_index(mk_var(xt, Type::pointer(c.sz)), fold_expr(mk_binop(BinOp::Add, mk_binop(BinOp::Mul, ce, mk_int(c.K, isz), ity), de, ity)), elem);
+    S inner = mk_for(dv, mk_int(0, isz), mk_int(c.K, isz), 1, {mk_assign(dst, src)}, LoopPar());
+    LoopPar par;
+    par.nthreads = c.N;
+    par.tpb = 256;
+    auto outer = std::const_pointer_cast<Stmt>(std::static_pointer_cast<const Stmt>(mk_for(cv, mk_int(0, isz), mk_int(c.N, isz), 1, {inner}, par)));
+    int64_t n = (c.N + WAVE_SIZE - 1) / WAVE_SIZE * WAVE_SIZE;
+    Kernel k;
+    k.name = p.name + "_transpose_" + x.s + "_" + std::to_string(gen.next++);
+    if (n > 256) {
+      outer->map.k = GpuMap::ThreadBlock;
+      outer->map.n = n;
+      outer->map.tpb = 256;
+      k.grid.x = (n + 255) / 256;
+      k.block.x = 256;
+    } else {
+      outer->map.k = GpuMap::Thread;
+      outer->map.n = n;
+      k.block.x = n;
+    }
+    outer->map.dim = 0;
+    k.body = {S(outer)};
+    KernelParam px, pxt;
+    px.id = x;
+    px.ty = Type::pointer(c.sz);
+    pxt.id = xt;
+    pxt.ty = Type::pointer(c.sz);
+    k.params = {px, pxt};
+    return k;
+  }
+
+  void run() {
+    Stmts host;
+    std::vector<Kernel> extra;
+    for (auto& s : p.host) {
+      if (s->k != Stmt::Launch) { host.push_back(s); continue; }
+      Kernel* k = nullptr;
+      for (auto& kk : p.kernels)
+        if (kk.name == s->fname) k = &kk;
+      if (!k) { host.push_back(s); continue; }
+      std::map<Name, Cand> cands;
+      std::set<Name> written;
+      visit_stmts(k->body, [&](const S& st) {
+        if (st->k == Stmt::Assign && st->dst->k == Expr::Index)
+          visit_exprs(st->dst->args[0], [&](const E& x) { if (x->k == Expr::Var) written.insert(x->name); });
+        if ((st->k == Stmt::Def && !st->ty.is_scalar()) || (st->k == Stmt::Assign && st->dst->k == Expr::Var && !st->dst->ty.is_scalar()))
+          visit_exprs(st->expr, [&](const E& x) { if (x->k == Expr::Var) written.insert(x->name); });  // aliased: leave alone
+      });
+      for (auto& q : k->params)
+        if (q.ty.is_pointer() && !written.count(q.id)) { Cand c; c.arr = q.id; cands[q.id] = c; }
+      std::vector<std::pair<Name, int64_t>> seq_loops;
+      scan(k->body, seq_loops, cands);
+      std::map<Name, Name> staged;
+      Stmts pre, post;
+      for (auto& kv : cands) {
+        const Cand& c = kv.second;
+        // worth it when the stride is at least a cache line and the matrix is re-read many times
+        if (!c.ok || !c.seen || c.N < 32 || c.K < 8 || c.K * c.N * elem_bytes(c.sz) > (int64_t(1) << 30)) continue;
+        Name xt = gen.fresh(c.arr.s + "_T");
+        staged[c.arr] = xt;
+        auto a = std::make_shared<Stmt>();
+        a->k = Stmt::Alloc;
+        a->id = xt;
+        a->ty = Type::scalar(c.sz);
+        a->iv = c.K * c.N;
+        pre.push_back(a);
+        Kernel tk = make_transpose(c.arr, xt, c);
+        auto l = std::make_shared<Stmt>();
+        l->k = Stmt::Launch;
+        l->fname = tk.name;
+        l->grid = tk.grid;
+        l->block = tk.block;
+        // the launch argument is whatever the consumer was given for this parameter
+        E src_arg;
+        for (size_t i = 0; i < k->params.size(); ++i)
+          if (k->params[i].id == c.arr) src_arg = s->args[i];
+        l->args = {src_arg, mk_var(xt, Type::pointer(c.sz))};
+        pre.push_back(l);
+        extra.push_back(tk);
+        auto f = std::make_shared<Stmt>();
+        f->k = Stmt::Free;
+        f->id = xt;
+        post.push_back(f);
+      }
+      if (staged.empty()) { host.push_back(s); continue; }
+      Type ity = Type::scalar(isz);
+      k->body = rewrite_stmts(k->body, [&](const E& e) -> E {
+        if (e->k == Expr::Index && e->args[0]->k == Expr::Var && staged.count(e->args[0]->name)) {
+          const Cand& c = cands[e->args[0]->name];
+          auto n = std::make_shared<Expr>(*e);
+          E idx = fold_expr(mk_binop(BinOp::Add, mk_binop(BinOp::Mul, e->dim_idx[1], mk_int(c.K, isz), ity), e->dim_idx[0], ity));
+          n->args = {mk_var(staged.at(e->args[0]->name), Type::tensor(c.sz, {c.N, c.K}), e->i), idx};
+          n->dim_idx = {e->dim_idx[1], e->dim_idx[0]};
+          n->dim_shape = {c.N, c.K};
+          return n;
+        }
+        return e;
+      });
+      auto ns = std::make_shared<Stmt>(*s);
+      for (size_t i = 0; i < k->params.size(); ++i)
+        if (staged.count(k->params[i].id)) {
+          Name xt = staged.at(k->params[i].id);
+          ns->args[i] = mk_var(xt, Type::pointer(k->params[i].ty.sz));
+          k->params[i].id = xt;
+        }
+      for (auto& q : pre) host.push_back(q);
+      host.push_back(ns);
+      for (auto& q : post) host.push_back(q);
+    }
+    for (auto& e : extra) p.kernels.push_back(e);
+    p.host = host;
+  }
+};
+
 }  // namespace
 
 void hip_optimize(Program& p, const Options& opts, NameGen& gen) {
+  if (opts.opt_gather_transpose) GatherTranspose(p, opts, gen).run();
   for (auto& k : p.kernels) {
     Pass pass(k, opts, gen);
     if (opts.opt_unswitch) pass.unswitch_aliases();
@@ -986,6 +1207,7 @@ void hip_optimize(Program& p, const Options& opts, NameGen& gen) {
     if (opts.opt_hoist_invariant) k.body = pass.hoist_invariant(k.body, &budget, false);
     if (opts.opt_reg_cache) pass.reg_cache(&budget);
     pass.mark_read_only();
+    if (opts.opt_nontemporal) pass.mark_streaming_loads();
     k.aligned_params = opts.assume_aligned;
   }
 }

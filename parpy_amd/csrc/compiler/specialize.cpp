@@ -82,6 +82,8 @@ Options parse_options(const std::string& sexpr) {
     else if (h == "opt_narrow_index") o.opt_narrow_index = flag();
     else if (h == "opt_mfma_sddmm") o.opt_mfma_sddmm = flag();
     else if (h == "opt_unswitch") o.opt_unswitch = flag();
+    else if (h == "opt_nontemporal") o.opt_nontemporal = flag();
+    else if (h == "opt_gather_transpose") o.opt_gather_transpose = flag();
     else if (h == "reg_budget") o.reg_budget = f->at(1)->as_int();
     else if (h == "assume_aligned") o.assume_aligned = flag();
     else if (h == "backend") {

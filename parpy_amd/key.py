@@ -31,5 +31,5 @@ def _generate_fast_cache_key(ir_ast, args, opts):
     from .compiler import print_ast
     extra = [getattr(opts, n, None) for n in ("opt_vectorize", "opt_lds_rows", "opt_reg_cache",
                                               "opt_hoist_invariant", "opt_narrow_index", "opt_mfma_sddmm",
-                                              "opt_unswitch", "assume_aligned", "reg_budget")]
+                                              "opt_unswitch", "opt_gather_transpose", "opt_nontemporal", "assume_aligned", "reg_budget")]
     return f"{print_ast(ir_ast)}+{_print_arguments_key(args)}+{opts}+{extra}"
