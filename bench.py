@@ -82,6 +82,7 @@ def bench_hmm(k, args, torch, parpy, W):
 def bench_rowsum(args, torch, parpy, W):
     import numpy as np
     N, M = 1024, 65536
+    args.inner_threads = args.inner_threads or 256   # 4 workgroups per CU overlap their load and reduce phases
     x = W.make_rowsum(N, M)
     xd = torch.from_numpy(x).cuda()
     out = torch.zeros(N, dtype=torch.float32, device="cuda")
@@ -111,6 +112,7 @@ def bench_rowsum(args, torch, parpy, W):
 def bench_softmax(args, torch, parpy, W):
     import numpy as np
     N, M = 16384, 4096
+    args.inner_threads = args.inner_threads or 512   # 8 elements (two dwordx4) per thread, 4 workgroups per CU
     x = W.make_softmax(N, M)
     xd = x.cuda()
     out = torch.zeros_like(xd)
@@ -219,7 +221,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--workload", default="hmm7", choices=["hmm7", "hmm5", "rowsum", "softmax", "sddmm", "copy"])
     ap.add_argument("--state-threads", type=int, default=1024)
-    ap.add_argument("--inner-threads", type=int, default=1024)
+    ap.add_argument("--inner-threads", type=int, default=None)
     ap.add_argument("--tpb", type=int, default=256)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-steps", type=int, default=0, help="samples per read for the HMM CPU baseline")

@@ -35,6 +35,28 @@ def _check_array_interface(intf):
     return shape, dtype, data
 
 
+_TORCH_DTYPES = {}
+
+
+def _torch_tensor_info(t):
+    """(shape, dtype, device pointer) of a plain torch tensor on the device without going through
+    its array-interface property (which builds a dict on every access), or None."""
+    import sys
+    torch = sys.modules.get("torch")
+    if torch is None or type(t) is not torch.Tensor or not t.is_cuda or t.requires_grad:
+        return None
+    if not t.is_contiguous():
+        raise ValueError("Buffers must only operate on contiguous memory")
+    if not _TORCH_DTYPES:
+        for sz in ElemSize:
+            dt = DataType.from_elem_size(sz)
+            _TORCH_DTYPES.setdefault(dt.to_torch(), dt)
+    dtype = _TORCH_DTYPES.get(t.dtype)
+    if dtype is None:
+        return None
+    return tuple(t.shape), dtype, t.data_ptr()
+
+
 def _to_array_interface(ptr, dtype, shape):
     return {"data": (ptr, False), "strides": None, "typestr": str(dtype), "shape": shape, "version": 3}
 
@@ -214,24 +236,30 @@ class DummyBuffer(Buffer):
 class HipBuffer(Buffer):
     """A torch tensor on the ROCm device, shared zero-copy with generated kernels."""
 
-    def __init__(self, buf, shape, dtype, src=None, refcount=None):
+    def __init__(self, buf, shape, dtype, src=None, refcount=None, ptr=None):
         super().__init__(buf, shape, dtype, src, refcount)
-        self.__cuda_array_interface__ = buf.__cuda_array_interface__
+        self._ptr = ptr
         self.backend = CompileBackend.Hip
         self.lib = _compile_runtime_lib(self.backend)
 
+    @property
+    def __cuda_array_interface__(self):
+        return self.buf.__cuda_array_interface__
+
     def _deconstruct(self, src_ptr):
         if src_ptr is not None:
-            _, _, buf_ptr = _extract_array_interface(self.buf, allow_cuda=True)
-            _check_errors(self.lib, self.lib.parpy_memcpy(src_ptr, buf_ptr, self.size(), 2))
+            _check_errors(self.lib, self.lib.parpy_memcpy(src_ptr, self._get_ptr(), self.size(), 2))
             self.sync()
 
     @staticmethod
     def _from_array(t):
+        info = _torch_tensor_info(t)
+        if info is not None:
+            return HipBuffer(t, info[0], info[1], ptr=info[2])
         try:
             shape, dtype, data_ptr = _extract_array_interface(t, allow_cuda=True)
             if hasattr(t, "__cuda_array_interface__"):
-                return HipBuffer(t, shape, dtype)
+                return HipBuffer(t, shape, dtype, ptr=data_ptr)
         except ValueError:
             raise ValueError(f"Cannot convert argument {t} to a HIP buffer")
         import torch
@@ -244,11 +272,12 @@ class HipBuffer(Buffer):
         _check_errors(lib, lib.parpy_memcpy(ptr, data_ptr, _size(shape, dtype), 1))
         # the host-to-device copy is asynchronous: the source must outlive it
         _check_errors(lib, lib.parpy_sync())
-        return HipBuffer(data, shape, dtype, src=t)
+        return HipBuffer(data, shape, dtype, src=t, ptr=ptr)
 
     def _get_ptr(self):
-        _, _, ptr = _extract_array_interface(self.buf, allow_cuda=True)
-        return ptr
+        if self._ptr is None:
+            _, _, self._ptr = _extract_array_interface(self.buf, allow_cuda=True)
+        return self._ptr
 
     def numpy(self):
         import numpy as np
@@ -261,15 +290,17 @@ class HipBuffer(Buffer):
         return HipBuffer(self.buf.detach().clone(), self.shape, self.dtype)
 
     def reshape(self, *dims):
-        b = super().reshape(*dims)
-        b.buf = b.buf.reshape(b.shape)
-        return b
+        import math
+        new_shape = tuple(dims)
+        if math.prod(self.shape) != math.prod(new_shape):
+            raise ValueError(f"Cannot reshape buffer of shape {self.shape} to {new_shape}")
+        return HipBuffer(self.buf.reshape(new_shape), new_shape, self.dtype, self.src, self.refcount, self._ptr)
 
     def with_type(self, new_dtype):
         new_dtype = _resolve_dtype(new_dtype)
         if isinstance(new_dtype, DataType):
             if self.dtype.size() == new_dtype.size():
-                return HipBuffer(self.buf, self.shape, new_dtype, self.src, self.refcount)
+                return HipBuffer(self.buf, self.shape, new_dtype, self.src, self.refcount, self._ptr)
             t = self.buf.detach().clone().to(new_dtype.to_torch())
             return HipBuffer(t, self.shape, new_dtype)
         raise ValueError(f"Found unsupported data type: {type(new_dtype)}")

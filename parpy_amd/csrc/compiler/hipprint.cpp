@@ -364,7 +364,6 @@ struct DevicePrinter {
         }
         std::string out = pexpr(e->args[0]) + "[" + pexpr(e->args[1]) + "]";
         for (auto& n : assumed) ranges.erase(n);
-        if (e->bv) return "__builtin_nontemporal_load(&" + out + ")";  // read-once data (marked by the optimiser)
         return out;
       }
       case Expr::AddrOf: return "(&" + pexpr(e->args[0]) + "[" + pexpr(e->args[1]) + "])";

@@ -27,9 +27,21 @@ def _print_arguments_key(args):
     return "-".join(_print_argument_key(arg) for arg in args)
 
 
+_ast_keys = {}
+
+
+def _ast_key(ir_ast):
+    """Printed form of a parsed function; it never changes after parsing, so it is printed once."""
+    k = _ast_keys.get(id(ir_ast))
+    if k is None or k[0] is not ir_ast:
+        from .compiler import print_ast
+        k = _ast_keys[id(ir_ast)] = (ir_ast, print_ast(ir_ast))
+    return k[1]
+
+
 def _generate_fast_cache_key(ir_ast, args, opts):
-    from .compiler import print_ast
     extra = [getattr(opts, n, None) for n in ("opt_vectorize", "opt_lds_rows", "opt_reg_cache",
                                               "opt_hoist_invariant", "opt_narrow_index", "opt_mfma_sddmm",
                                               "opt_unswitch", "opt_gather_transpose", "opt_nontemporal", "assume_aligned", "reg_budget")]
-    return f"{print_ast(ir_ast)}+{_print_arguments_key(args)}+{opts}+{extra}"
+    # a tuple: the (long) printed function keeps its cached hash from one call to the next
+    return (_ast_key(ir_ast), _print_arguments_key(args), str(opts), tuple(extra))

@@ -322,3 +322,14 @@ def test_unaligned_views_get_their_own_specialisation():
     W.copy_1d(x, out, opts=opts_for({'N': parpy.threads(N // 4)}))
     parpy.sync(HIP)
     assert torch.equal(out, x)
+
+
+@pytest.mark.parametrize("n,threads,tpb", [(1 << 20, 1 << 16, 256), (1 << 20, 1 << 18, 1024), (1000, 100, 64), (4096 + 64, 256, 64)])
+def test_grid_wide_elementwise_loop(n, threads, tpb):
+    """A grid-mapped element-wise loop: four consecutive elements per thread where the launch has
+    no partial block and the extent divides evenly, the plain strided form elsewhere."""
+    x = torch.arange(n, dtype=torch.float32, device="cuda") * 0.5
+    out = torch.zeros_like(x)
+    W.copy_1d(x, out, opts=opts_for({'N': parpy.threads(threads).tpb(tpb)}))
+    parpy.sync(HIP)
+    assert torch.equal(out, x)
