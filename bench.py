@@ -46,6 +46,7 @@ def bench_hmm(k, args, torch, parpy, W):
     nthreads = min(S, args.state_threads)
     opts = parpy.par({"inst": parpy.threads(n), "state": parpy.threads(nthreads)})
     _apply_opt_flags(opts, args)
+    opts.use_cuda_graphs = bool(args.use_graphs)
     fn = lambda: W.forward_syn(hd, sd, res, a1, a2, opts=opts)
     timed = lambda: parpy.time_call(W.forward_syn, hd, sd, res, a1, a2, opts=opts)
     wall, dev = _events_ms(fn, timed, args.steps, args.warmup, torch)
@@ -70,7 +71,7 @@ def bench_hmm(k, args, torch, parpy, W):
         "value": wall, "unit": "ms/batch", "ms_per_step": wall, "higher_is_better": False,
         "dtype": "f32",
         "config": {"workload": f"hmm_forward_{k}mer_synthetic", "states": S, "reads": n, "min_len": 5000,
-                   "max_len": 15000, "total_steps": steps_total, "state_threads": nthreads,
+                   "max_len": 15000, "total_steps": steps_total, "state_threads": nthreads, "graph_replay": bool(args.use_graphs),
                    "mean_loglik": float(ll.mean())},
         "roofline": {"bound": "hbm", "achieved": alg_bytes / (kernel_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": alg_bytes / (kernel_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None,
@@ -206,7 +207,7 @@ def _profiled_traffic(name):
 
 
 def _apply_opt_flags(opts, args):
-    for name in ("opt_vectorize", "opt_lds_rows", "opt_reg_cache", "opt_hoist_invariant", "opt_narrow_index", "opt_unswitch", "opt_gather_transpose", "opt_nontemporal"):
+    for name in ("opt_vectorize", "opt_lds_rows", "opt_reg_cache", "opt_hoist_invariant", "opt_narrow_index", "opt_unswitch", "opt_gather_transpose", "opt_nontemporal", "opt_mfma_sddmm"):
         v = getattr(args, name)
         if v is not None:
             setattr(opts, name, bool(v))
@@ -221,11 +222,12 @@ def main():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--workload", default="hmm7", choices=["hmm7", "hmm5", "rowsum", "softmax", "sddmm", "copy"])
     ap.add_argument("--state-threads", type=int, default=1024)
+    ap.add_argument("--use-graphs", type=int, default=0, help="replay the launches of a run from a HIP graph (host-hoisted time loops)")
     ap.add_argument("--inner-threads", type=int, default=None)
     ap.add_argument("--tpb", type=int, default=256)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-steps", type=int, default=0, help="samples per read for the HMM CPU baseline")
-    for name in ("opt_vectorize", "opt_lds_rows", "opt_reg_cache", "opt_hoist_invariant", "opt_narrow_index", "opt_unswitch", "opt_gather_transpose", "opt_nontemporal"):
+    for name in ("opt_vectorize", "opt_lds_rows", "opt_reg_cache", "opt_hoist_invariant", "opt_narrow_index", "opt_unswitch", "opt_gather_transpose", "opt_nontemporal", "opt_mfma_sddmm"):
         ap.add_argument("--" + name.replace("_", "-"), dest=name, type=int, default=None)
     ap.add_argument("--reg-budget", type=int, default=0)
     args = ap.parse_args()
@@ -254,7 +256,7 @@ def main():
     else:
         r = bench_sddmm(args, torch, parpy, W)
     default_cfg = not any(getattr(args, n) is not None for n in ("opt_vectorize", "opt_lds_rows", "opt_reg_cache",
-                                                                 "opt_hoist_invariant", "opt_narrow_index", "opt_unswitch", "opt_gather_transpose", "opt_nontemporal"))
+                                                                 "opt_hoist_invariant", "opt_narrow_index", "opt_unswitch", "opt_gather_transpose", "opt_nontemporal", "opt_mfma_sddmm"))
     if default_cfg and not args.reg_budget:
         r["roofline"]["traffic"] = _profiled_traffic(args.workload)
     r.update({"n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "scaling": "weak", "vs_baseline": None,

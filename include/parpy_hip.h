@@ -80,6 +80,19 @@ int32_t parpy_hip_plan_run(void* plan, void* const* args, int32_t nargs);
 int32_t parpy_hip_plan_run_timed(void* plan, void* const* args, int32_t nargs,
                                  float* elapsed_ms);
 
+/* Graph replay for plans whose host side is a long loop of launches: the
+ * analogue of the reference's use_cuda_graphs option (src/option.rs:60-63,
+ * src/cuda/graphs.rs).  With it enabled the first run is eager (it allocates
+ * the device temporaries), the second is captured into a HIP graph, and later
+ * runs with the same pointer arguments are one hipGraphLaunch on the null
+ * stream; other pointers trigger a new capture.  A plan that would have to
+ * allocate during capture falls back to eager launches. */
+int32_t parpy_hip_plan_set_graph(void* plan, int32_t enable);
+
+/* Number of runs of this plan that were served by a graph replay so far
+ * (0 for a plan that runs eagerly or that fell back). */
+int64_t parpy_hip_plan_graph_replays(void* plan);
+
 /* Number of kernel launches the last run of this plan enqueued. */
 int64_t parpy_hip_plan_launch_count(void* plan);
 

@@ -111,6 +111,9 @@ def get_wrapper(name, key, plan_text, opts):
     if rc != 0:
         raise RuntimeError(lib.parpy_get_error_message().decode("ascii", "replace"))
 
+    if opts.use_cuda_graphs:
+        lib.parpy_hip_plan_set_graph(plan, 1)
+
     def wrapper(*args):
         flat = [x for a in args for x in _expand_arg(a)]
         # scalars and 0-d buffers were folded into the code; what is passed are array pointers
@@ -135,6 +138,7 @@ def get_wrapper(name, key, plan_text, opts):
     wrapper.timed = timed
     wrapper.plan = plan
     wrapper.launch_count = lambda: lib.parpy_hip_plan_launch_count(plan)
+    wrapper.graph_replays = lambda: lib.parpy_hip_plan_graph_replays(plan)
     return wrapper
 
 
@@ -148,6 +152,9 @@ def get_string_wrapper(kernel_name, key, grid, block, opts):
     sizes = ScalarSizes(opts)
     g = (ctypes.c_int64 * 3)(*grid)
     b = (ctypes.c_int64 * 3)(*block)
+
+    if opts.use_cuda_graphs:
+        lib.parpy_hip_plan_set_graph(plan, 1)
 
     def wrapper(*args):
         flat = [x for a in args for x in _expand_arg(a)]

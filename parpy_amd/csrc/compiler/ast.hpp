@@ -360,7 +360,7 @@ struct Options {  // src/option.rs:14-108
   bool opt_reg_cache = true;
   bool opt_hoist_invariant = true;
   bool opt_narrow_index = true;
-  bool opt_mfma_sddmm = true;
+  bool opt_mfma_sddmm = false;  // per-thread dot products on the matrix cores (4x4x1 tiles): measured slower, opt-in
   bool opt_unswitch = false;   // measured slower on the HMM kernels (higher register pressure): opt-in
   bool opt_gather_transpose = true;
   bool opt_nontemporal = true;   // non-temporal stores to arrays a kernel only writes
@@ -384,6 +384,8 @@ struct Kernel {
   Dim3 grid, block;
   int64_t lds_bytes = 0;
   bool aligned_params = false;  // every pointer argument is 16-byte aligned (checked by the caller)
+  bool cached_stores = false;   // what this kernel writes is read by the next one: no non-temporal stores
+  bool opaque_body = false;     // the body is a call of a device helper: parameters are described by the creator
 };
 
 struct Program {

@@ -947,6 +947,56 @@ struct Pass {
     k.body = {nr};
   }
 
+  // ================================================================ dot products on the matrix cores
+  // `t = t + X[..] * Y[..]` in an innermost sequential f32 loop of constant length is a dot
+  // product that every thread computes for itself.  v_mfma_f32_4x4x1 multiplies, for each group
+  // of four lanes, the four X values by the four Y values of the group (a 4 x 4 outer product
+  // accumulated over the loop); the product a thread wants is element [lane % 4] of its own
+  // column.  Three quarters of the multiplications are thrown away and the instruction takes two
+  // passes, so this is no faster than v_fmac on the vector ALU: there is no operand reuse between
+  // the dot products of different threads for a matrix unit to exploit.  Kept as an option so
+  // that the comparison can be measured.
+  Stmts mfma_dot(const Stmts& ss) {
+    Stmts out;
+    for (auto& s : ss) {
+      bool inner = s->k == Stmt::For && s->map.k == GpuMap::None && s->step == 1 && s->hi->k == Expr::Int && s->lo->k == Expr::Int &&
+                   s->body.size() == 1 && s->body[0]->k == Stmt::Assign && s->body[0]->dst->k == Expr::Var;
+      if (inner) {
+        const S& a = s->body[0];
+        const E& t = a->dst;
+        E mul;
+        if (a->expr->k == Expr::BinOpE && a->expr->bop == BinOp::Add) {
+          const E &l = a->expr->args[0], &r = a->expr->args[1];
+          if (l->k == Expr::Var && l->name == t->name) mul = r;
+          else if (r->k == Expr::Var && r->name == t->name) mul = l;
+        }
+        bool ok = mul && mul->k == Expr::BinOpE && mul->bop == BinOp::Mul && t->ty.is_scalar() && t->ty.sz == ElemSize::F32 &&
+                  mul->args[0]->k == Expr::Index && mul->args[1]->k == Expr::Index && mul->args[0]->ty.sz == ElemSize::F32 &&
+                  mul->args[1]->ty.sz == ElemSize::F32 && !mentions(mul, t->name);
+        if (ok) {
+          Name acc = gen.fresh(t->name.s + "_acc");
+          Type f32 = Type::scalar(ElemSize::F32);
+          out.push_back(mk_rawstmt("parpy_f32x4 " + acc.str() + " = {0.0f, 0.0f, 0.0f, 0.0f};"));
+          auto call = std::make_shared<Expr>();
+          call->k = Expr::Call;
+          call->ty = f32;
+          call->sval = "__builtin_amdgcn_mfma_f32_4x4x1f32";
+          call->args = {mul->args[0], mul->args[1], mk_var(acc, f32), mk_raw("0", f32), mk_raw("0", f32), mk_raw("0", f32)};
+          auto loop = clone(s);
+          loop->body = {mk_assign(mk_var(acc, f32), call)};
+          out.push_back(loop);
+          out.push_back(mk_assign(t, mk_binop(BinOp::Add, t, mk_raw(acc.str() + "[parpy_lane_id() & 3]", f32), f32)));
+          continue;
+        }
+      }
+      auto r = clone(s);
+      r->body = mfma_dot(s->body);
+      r->els = mfma_dot(s->els);
+      out.push_back(r);
+    }
+    return out;
+  }
+
   // ================================================================ read-only parameters
   // A pointer parameter is read-only when nothing in the kernel stores through
   // it, directly or through a local alias initialised from it.
@@ -1030,6 +1080,27 @@ struct GatherTranspose {
   }
 
   Kernel make_transpose(const Name& x, const Name& xt, const Cand& c) {
+    KernelParam px, pxt;
+    px.id = x;
+    px.ty = Type::pointer(c.sz);
+    px.read_only = true;
+    pxt.id = xt;
+    pxt.ty = Type::pointer(c.sz);
+    if (c.K % 64 == 0 && c.N % 64 == 0 && elem_bytes(c.sz) >= 4) {
+      // whole 64 x 64 tiles: turned round in LDS by a device helper, whole lines on both sides
+      Kernel k;
+      k.name = p.name + "_transpose_" + x.s + "_" + std::to_string(gen.next++);
+      k.grid.x = c.N / 64;
+      k.grid.y = c.K / 64;
+      k.block.x = 256;
+      k.lds_bytes = 64 * 65 * elem_bytes(c.sz);
+      k.cached_stores = true;
+      k.opaque_body = true;
+      k.body = {mk_rawstmt("parpy_transpose_tile<" + std::string(elem_ctype(c.sz)) + ", " + std::to_string(c.K) + ", " +
+                           std::to_string(c.N) + ">(" + x.str() + ", " + xt.str() + ");")};
+      k.params = {px, pxt};
+      return k;
+    }
     // one thread per column c; reads are coalesced across the wavefront, each thread writes its own row of X^T
     Type ity = Type::scalar(isz);
     Type elem = Type::scalar(c.sz);
@@ -1058,11 +1129,7 @@ struct GatherTranspose {
     }
     outer->map.dim = 0;
     k.body = {S(outer)};
-    KernelParam px, pxt;
-    px.id = x;
-    px.ty = Type::pointer(c.sz);
-    pxt.id = xt;
-    pxt.ty = Type::pointer(c.sz);
+    k.cached_stores = true;
     k.params = {px, pxt};
     return k;
   }
@@ -1155,8 +1222,10 @@ struct GatherTranspose {
 void hip_optimize(Program& p, const Options& opts, NameGen& gen) {
   if (opts.opt_gather_transpose) GatherTranspose(p, opts, gen).run();
   for (auto& k : p.kernels) {
+    if (k.opaque_body) { k.aligned_params = opts.assume_aligned; continue; }
     Pass pass(k, opts, gen);
     if (opts.opt_unswitch) pass.unswitch_aliases();
+    if (opts.opt_mfma_sddmm) k.body = pass.mfma_dot(k.body);
     if (opts.opt_lds_rows) pass.lds_rows();
     if (opts.opt_vectorize) k.body = pass.vectorize(k.body);
     int64_t budget = pass.reg_budget();

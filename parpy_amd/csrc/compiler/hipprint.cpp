@@ -146,6 +146,21 @@ __device__ __forceinline__ T parpy_block_reduce(T v, T neutral, T* slots, bool s
   }
   return v;
 }
+typedef float parpy_f32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ int parpy_lane_id() { return (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)); }
+// dst[c][r] = src[r][c] for a ROWS x COLS matrix in 64 x 64 tiles: a 256-thread workgroup reads
+// 64-word row segments of its tile, turns the tile round in LDS and writes 64-word row segments
+// of the result, so both sides move whole 256-byte lines.  Launched on a (COLS/64, ROWS/64) grid.
+template <class T, int ROWS, int COLS> __device__ __forceinline__ void parpy_transpose_tile(const T* __restrict__ src, T* __restrict__ dst) {
+  __shared__ T tile[64][65];
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  const int c0 = (int)blockIdx.x * 64, r0 = (int)blockIdx.y * 64;
+  #pragma unroll
+  for (int j = 0; j < 16; ++j) tile[j * 4 + ty][tx] = src[(long long)(r0 + j * 4 + ty) * COLS + c0 + tx];
+  __syncthreads();
+  #pragma unroll
+  for (int j = 0; j < 16; ++j) dst[(long long)(c0 + j * 4 + ty) * ROWS + r0 + tx] = tile[tx][j * 4 + ty];
+}
 )";
 
 struct PE {  // printed integer expression: text + whether it was computed in 32-bit arithmetic
@@ -370,6 +385,11 @@ struct DevicePrinter {
       case Expr::ThreadIdx: case Expr::BlockIdx: return "((int64_t)" + idx_name(e->k, (int)e->iv) + ")";
       case Expr::RegElem: return e->name.str() + "[" + pexpr(e->args[0]) + "]";
       case Expr::Raw: return e->sval;
+      case Expr::Call: {
+        std::string out = e->sval + "(";
+        for (size_t a = 0; a < e->args.size(); ++a) out += (a ? ", " : "") + pexpr(e->args[a]);
+        return out + ")";
+      }
       default: fail_rt(e->i, "Cannot print expression " + print_expr(e) + " (internal error)");
     }
   }
@@ -455,7 +475,7 @@ struct DevicePrinter {
       os << ind(n + 2) << vty << " " << v << " = " << init(idx) << ";\n";
       std::string cond;
       if (extent < launched) cond = v + cmp + his;
-      if (!guard.empty()) cond = cond.empty() ? guard : cond + " && " + guard;
+      if (!guard.empty() && cond.empty()) cond = guard;  // v < hi already implies the launch guard (extent <= N)
       if (!cond.empty()) {
         os << ind(n + 2) << "if (" << cond << ") {\n";
         pstmts(s->body, n + 4);
@@ -584,7 +604,7 @@ struct DevicePrinter {
     os.str("");
     find_reassigned(k.body, reassigned);
     stream_out.clear();
-    if (opts.opt_nontemporal) {
+    if (opts.opt_nontemporal && !k.cached_stores) {
       // parameters that are stored to (directly, never through an alias) and never read in this kernel
       std::set<Name> read, aliased;
       visit_stmts(k.body, [&](const S& st) {

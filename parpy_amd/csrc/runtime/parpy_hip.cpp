@@ -88,6 +88,8 @@ struct HStmt {
   std::vector<HStmt> body, els;
 };
 
+constexpr int64_t KEEP_LIMIT = int64_t(1) << 30;
+
 struct Plan {
   hipModule_t module = nullptr;
   std::vector<hipFunction_t> fns;
@@ -98,7 +100,25 @@ struct Plan {
   std::vector<HStmt> body;
   std::vector<Val> env;
   int64_t launches = 0;
+  // Device temporaries stay allocated between runs of the plan (up to KEEP_LIMIT bytes per plan):
+  // a run then costs no allocator call.  Indexed by variable slot.
+  struct Kept { void* ptr = nullptr; int64_t nbytes = 0; bool in_use = false; };
+  std::vector<Kept> kept;
+  int64_t kept_bytes = 0;
   hipEvent_t ev_start = nullptr, ev_stop = nullptr;  // created on the first timed run
+  // Graph replay (the analogue of the reference's use_cuda_graphs, src/cuda/graphs.rs): the
+  // launches of one run are captured into a HIP graph and later runs with the same pointer
+  // arguments replay it with a single hipGraphLaunch.
+  bool use_graph = false;
+  int graph_state = 0;                 // 0 = first run still to come (eager, allocates the temporaries), 1 = usable, -1 = given up
+  hipStream_t cap_stream = nullptr;    // capture needs a stream of its own; replays go to the null stream
+  hipStream_t launch_stream = nullptr; // where run_stmt enqueues: null stream, or cap_stream while capturing
+  bool capturing = false;
+  hipGraph_t graph = nullptr;
+  hipGraphExec_t graph_exec = nullptr;
+  std::vector<void*> graph_args;
+  int64_t graph_launches = 0;
+  int64_t graph_replays = 0;           // runs served by hipGraphLaunch so far
 };
 
 struct PlanBuilder {
@@ -350,7 +370,7 @@ int32_t run_stmt(Plan& p, const HStmt& s) {
       }
       ++p.launches;
       return check(hipModuleLaunchKernel(p.fns[s.kernel], s.grid[0], s.grid[1], s.grid[2], s.block[0], s.block[1],
-                                         s.block[2], 0, nullptr, ptrs, nullptr),
+                                         s.block[2], 0, p.launch_stream, ptrs, nullptr),
                    p.knames[s.kernel].c_str());
     }
     case HStmt::For: {
@@ -372,6 +392,15 @@ int32_t run_stmt(Plan& p, const HStmt& s) {
       p.env[s.slot] = eval(p, s.a);
       return 0;
     case HStmt::Alloc: {
+      if (p.kept.size() < p.env.size()) p.kept.resize(p.env.size());
+      Plan::Kept& kp = p.kept[s.slot];
+      if (kp.ptr && kp.nbytes == s.nbytes && !kp.in_use) {
+        kp.in_use = true;
+        p.env[s.slot].t = Val::P;
+        p.env[s.slot].p = kp.ptr;
+        return 0;
+      }
+      if (p.capturing) return fail("a device temporary would have to be allocated inside a graph capture");
       void* ptr = nullptr;
       hipError_t e = hipMallocAsync(&ptr, (size_t)s.nbytes, nullptr);
       if (e != hipSuccess) {
@@ -381,11 +410,21 @@ int32_t run_stmt(Plan& p, const HStmt& s) {
       if (int32_t rc = check(e, "allocation of a device temporary")) return rc;
       p.env[s.slot].t = Val::P;
       p.env[s.slot].p = ptr;
+      if (!kp.ptr && p.kept_bytes + s.nbytes <= KEEP_LIMIT) {
+        kp.ptr = ptr;
+        kp.nbytes = s.nbytes;
+        kp.in_use = true;
+        p.kept_bytes += s.nbytes;
+      }
       return 0;
     }
     case HStmt::Free: {
       void* ptr = p.env[s.slot].p;
       p.env[s.slot].p = nullptr;
+      if ((size_t)s.slot < p.kept.size() && p.kept[s.slot].ptr == ptr && ptr) {
+        p.kept[s.slot].in_use = false;  // stays allocated for the next run
+        return 0;
+      }
       hipError_t e = hipFreeAsync(ptr, nullptr);
       if (e != hipSuccess) {
         (void)hipGetLastError();
@@ -542,6 +581,62 @@ int32_t parpy_hip_plan_create(void* module, const char* plan_text, void** plan) 
   return 0;
 }
 
+}  // extern "C"
+
+namespace {
+
+void drop_graph(Plan& p) {
+  if (p.graph_exec) (void)hipGraphExecDestroy(p.graph_exec);
+  if (p.graph) (void)hipGraphDestroy(p.graph);
+  p.graph_exec = nullptr;
+  p.graph = nullptr;
+}
+
+// Capture one run of the plan.  Returns false (and leaves graph_state = -1) when the plan cannot
+// be captured; the caller then runs it eagerly.
+bool capture_graph(Plan& p, void* const* args, int32_t nargs) {
+  drop_graph(p);
+  if (!p.cap_stream && hipStreamCreate(&p.cap_stream) != hipSuccess) {
+    (void)hipGetLastError();
+    p.graph_state = -1;
+    return false;
+  }
+  if (hipStreamBeginCapture(p.cap_stream, hipStreamCaptureModeThreadLocal) != hipSuccess) {
+    (void)hipGetLastError();
+    p.graph_state = -1;
+    return false;
+  }
+  p.launch_stream = p.cap_stream;
+  p.capturing = true;
+  p.launches = 0;
+  int32_t rc = run_stmts(p, p.body);
+  p.capturing = false;
+  p.launch_stream = nullptr;
+  hipError_t e = hipStreamEndCapture(p.cap_stream, &p.graph);
+  if (rc == 0 && e == hipSuccess) e = hipGraphInstantiate(&p.graph_exec, p.graph, nullptr, nullptr, 0);
+  if (rc != 0 || e != hipSuccess) {
+    (void)hipGetLastError();
+    drop_graph(p);
+    p.graph_state = -1;
+    return false;
+  }
+  p.graph_args.assign(args, args + nargs);
+  p.graph_launches = p.launches;
+  return true;
+}
+
+}  // namespace
+
+extern "C" {
+
+int32_t parpy_hip_plan_set_graph(void* plan, int32_t enable) {
+  Plan& p = *(Plan*)plan;
+  p.use_graph = enable != 0;
+  if (!p.use_graph) drop_graph(p);
+  p.graph_state = 0;
+  return 0;
+}
+
 int32_t parpy_hip_plan_run(void* plan, void* const* args, int32_t nargs) {
   Plan& p = *(Plan*)plan;
   if (nargs != p.nparams)
@@ -551,8 +646,20 @@ int32_t parpy_hip_plan_run(void* plan, void* const* args, int32_t nargs) {
     p.env[k].t = Val::P;
     p.env[k].p = args[k];
   }
+  for (auto& kp : p.kept) kp.in_use = false;  // a run that failed half way may have left a temporary marked
+  if (p.use_graph && p.graph_state == 1) {
+    bool same = p.graph_exec && p.graph_args.size() == (size_t)nargs && std::equal(args, args + nargs, p.graph_args.begin());
+    if (same || capture_graph(p, args, nargs)) {
+      p.launches = p.graph_launches;
+      ++p.graph_replays;
+      return check(hipGraphLaunch(p.graph_exec, nullptr), "hipGraphLaunch");
+    }
+    for (auto& kp : p.kept) kp.in_use = false;
+  }
   p.launches = 0;
-  return run_stmts(p, p.body);
+  int32_t rc = run_stmts(p, p.body);
+  if (p.use_graph && p.graph_state == 0) p.graph_state = rc == 0 ? 1 : -1;  // temporaries exist now: capture from the next run on
+  return rc;
 }
 
 int32_t parpy_hip_plan_run_timed(void* plan, void* const* args, int32_t nargs, float* elapsed_ms) {
@@ -570,10 +677,16 @@ int32_t parpy_hip_plan_run_timed(void* plan, void* const* args, int32_t nargs, f
 
 int64_t parpy_hip_plan_launch_count(void* plan) { return ((Plan*)plan)->launches; }
 
+int64_t parpy_hip_plan_graph_replays(void* plan) { return ((Plan*)plan)->graph_replays; }
+
 int32_t parpy_hip_plan_destroy(void* plan) {
   Plan* p = (Plan*)plan;
   if (p->ev_start) (void)hipEventDestroy(p->ev_start);
   if (p->ev_stop) (void)hipEventDestroy(p->ev_stop);
+  drop_graph(*p);
+  if (p->cap_stream) (void)hipStreamDestroy(p->cap_stream);
+  for (auto& kp : p->kept)
+    if (kp.ptr) (void)hipFree(kp.ptr);
   delete p;
   return 0;
 }

@@ -69,6 +69,10 @@ def init_library(libpath):
     lib.parpy_hip_plan_run.restype = i32
     lib.parpy_hip_plan_run_timed.argtypes = [vp, ctypes.POINTER(vp), i32, ctypes.POINTER(ctypes.c_float)]
     lib.parpy_hip_plan_run_timed.restype = i32
+    lib.parpy_hip_plan_set_graph.argtypes = [vp, i32]
+    lib.parpy_hip_plan_set_graph.restype = i32
+    lib.parpy_hip_plan_graph_replays.argtypes = [vp]
+    lib.parpy_hip_plan_graph_replays.restype = i64
     lib.parpy_hip_plan_launch_count.argtypes = [vp]
     lib.parpy_hip_plan_launch_count.restype = i64
     lib.parpy_hip_plan_destroy.argtypes = [vp]

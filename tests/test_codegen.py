@@ -179,6 +179,16 @@ def test_sddmm_kernels_compile():
     s0 = compiles(parpy.print_compiled(W.sddmm_coo, [A, B, C, np.zeros_like(vals), 1.5, 2.0],
                                        opts_for({"nnz": parpy.threads(len(cols))}, opt_gather_transpose=False)))
     assert launch(s0) == [("1", "1", "1", "832", "1", "1")]
+    # the matrix-core form of the per-thread dot product is opt-in
+    assert "mfma" not in s.split("extern \"C\" __global__", 1)[1]
+    sm = compiles(parpy.print_compiled(W.sddmm_coo, [A, B, C, np.zeros_like(vals), 1.5, 2.0],
+                                       opts_for({"nnz": parpy.threads(len(cols))}, opt_mfma_sddmm=True)))
+    assert "__builtin_amdgcn_mfma_f32_4x4x1f32(" in sm
+    # whole 64 x 64 tiles are transposed through LDS
+    A2, B2, crows2, cols2, vals2 = W.make_sddmm(256, 64, 0.05)
+    C2 = {"rows": oracle.csr_rows(crows2), "cols": cols2, "values": vals2, "nnz": len(cols2)}
+    st = compiles(parpy.print_compiled(W.sddmm_coo, [A2, B2, C2, np.zeros_like(vals2), 1.5, 2.0], opts_for({"nnz": parpy.threads(len(cols2))})))
+    assert "parpy_transpose_tile<float, 64, 256>(" in st and launch(st)[0] == ("4", "1", "1", "256", "1", "1")
     s = compiles(parpy.print_compiled(W.sddmm_decompress_csr, [crows, np.zeros_like(cols), 128],
                                       opts_for({"N": parpy.threads(128), "M": parpy.threads(64)})))
     assert launch(s) == [("1", "128", "1", "64", "1", "1")]

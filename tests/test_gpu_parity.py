@@ -215,8 +215,9 @@ def test_forward_all_states_unreachable_gives_neg_inf():
 
 
 # ---------------------------------------------------------------- SDDMM
+@pytest.mark.parametrize("flags", [{}, {"opt_mfma_sddmm": True}, {"opt_gather_transpose": False}], ids=["default", "mfma", "no-transpose"])
 @pytest.mark.parametrize("n,k,density", [(256, 32, 0.05), (8192, 128, 0.01)])
-def test_sddmm(n, k, density):
+def test_sddmm(n, k, density, flags):
     A, B, crows, cols, vals = W.make_sddmm(n, k, density)
     nnz = len(cols)
     Ad, Bd = torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda()
@@ -227,7 +228,7 @@ def test_sddmm(n, k, density):
     assert np.array_equal(rows_d.cpu().numpy(), rows)          # index work: bit-exact
     C = {"rows": rows_d, "cols": torch.from_numpy(cols).cuda(), "values": torch.from_numpy(vals).cuda(), "nnz": nnz}
     D = torch.zeros(nnz, dtype=torch.float32, device="cuda")
-    W.sddmm_coo(Ad, Bd, C, D, 1.5, 2.0, opts=opts_for({"nnz": parpy.threads(nnz).tpb(256)}))
+    W.sddmm_coo(Ad, Bd, C, D, 1.5, 2.0, opts=opts_for({"nnz": parpy.threads(nnz).tpb(256)}, **flags))
     want = oracle.sddmm(A, B, rows, cols, vals, alpha=1.5, beta=2.0)
     got = D.cpu().numpy()
     bad = np.abs(got - want) > 1e-5 + 1e-5 * np.abs(want)
@@ -333,3 +334,34 @@ def test_grid_wide_elementwise_loop(n, threads, tpb):
     W.copy_1d(x, out, opts=opts_for({'N': parpy.threads(threads).tpb(tpb)}))
     parpy.sync(HIP)
     assert torch.equal(out, x)
+
+
+def test_graph_replay_of_host_hoisted_time_loop():
+    """4096 states on 4096 threads need four workgroups per read, so the time loop runs on the host
+    (one launch per step).  With use_cuda_graphs the launches of a run are captured once and
+    replayed; every replay must give what the eager run gives, also after the program's own work
+    in between and after a change of buffers (which forces a new capture)."""
+    hmm, seqs = W.synthetic_hmm(6, n_inst=8, min_len=40, max_len=120)
+    want = oracle.hmm_syn_forward(hmm, seqs, np.float32)
+    hd, sd = W.to_device(hmm), W.to_device(seqs)
+    n, S = 8, 4096
+    sets = [[torch.zeros(n, dtype=torch.float32, device="cuda"), torch.zeros((n, S), dtype=torch.float32, device="cuda"),
+             torch.zeros((n, S), dtype=torch.float32, device="cuda")] for _ in range(2)]
+    o = opts_for({'inst': parpy.threads(n), 'state': parpy.threads(S)}, use_cuda_graphs=True)
+    eager = opts_for({'inst': parpy.threads(n), 'state': parpy.threads(S)})
+    for rep, which in enumerate([0, 0, 0, 0, 1, 1, 0]):   # eager, capture, replay, replay, re-capture, replay, re-capture
+        res, a1, a2 = sets[which]
+        for t in (res, a1, a2):
+            t.fill_(float(rep))
+        torch.cuda.synchronize()
+        W.forward_syn(hd, sd, res, a1, a2, opts=o)
+        got = res.cpu().numpy()
+        assert np.allclose(got, want, atol=1e-5, rtol=1e-5), (rep, np.abs(got - want).max())
+    res, a1, a2 = sets[0]
+    W.forward_syn(hd, sd, res, a1, a2, opts=eager)
+    assert np.allclose(res.cpu().numpy(), want, atol=1e-5, rtol=1e-5)
+    ms = parpy.time_call(W.forward_syn, hd, sd, res, a1, a2, opts=o)
+    assert 0 < ms < 1000
+    from parpy_amd import _fun_cache
+    replays = [w.graph_replays() for w in _fun_cache.values() if w.__name__ == "forward_syn"]
+    assert max(replays) >= 6 and max(w.launch_count() for w in _fun_cache.values() if w.__name__ == "forward_syn") >= 119
