@@ -57,7 +57,7 @@ def bench_hmm(k, args, torch, parpy, W):
     cpu = None
     if not args.no_cpu:
         import oracle
-        sample_steps = args.cpu_steps or (2000 if k <= 5 else 150)
+        sample_steps = args.cpu_steps or (15000 if k <= 5 else 5000)   # about 2 s (5-mer) and 10 s (7-mer) on 16 cores
         t0 = time.perf_counter()
         oracle.hmm_syn_forward(hmm, seqs, np.float32, max_steps=sample_steps)
         dt = time.perf_counter() - t0
@@ -207,7 +207,7 @@ def _profiled_traffic(name):
 
 
 def _apply_opt_flags(opts, args):
-    for name in ("opt_vectorize", "opt_lds_rows", "opt_reg_cache", "opt_hoist_invariant", "opt_narrow_index", "opt_unswitch", "opt_gather_transpose", "opt_nontemporal", "opt_mfma_sddmm"):
+    for name in ("opt_vectorize", "opt_lds_rows", "opt_reg_cache", "opt_hoist_invariant", "opt_narrow_index", "opt_unswitch", "opt_gather_transpose", "opt_nontemporal", "opt_noalias_scopes", "opt_mfma_sddmm"):
         v = getattr(args, name)
         if v is not None:
             setattr(opts, name, bool(v))
@@ -218,8 +218,8 @@ def _apply_opt_flags(opts, args):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=5)
-    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="hmm7", choices=["hmm7", "hmm5", "rowsum", "softmax", "sddmm", "copy"])
     ap.add_argument("--state-threads", type=int, default=1024)
     ap.add_argument("--use-graphs", type=int, default=0, help="replay the launches of a run from a HIP graph (host-hoisted time loops)")
@@ -227,7 +227,7 @@ def main():
     ap.add_argument("--tpb", type=int, default=256)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-steps", type=int, default=0, help="samples per read for the HMM CPU baseline")
-    for name in ("opt_vectorize", "opt_lds_rows", "opt_reg_cache", "opt_hoist_invariant", "opt_narrow_index", "opt_unswitch", "opt_gather_transpose", "opt_nontemporal", "opt_mfma_sddmm"):
+    for name in ("opt_vectorize", "opt_lds_rows", "opt_reg_cache", "opt_hoist_invariant", "opt_narrow_index", "opt_unswitch", "opt_gather_transpose", "opt_nontemporal", "opt_noalias_scopes", "opt_mfma_sddmm"):
         ap.add_argument("--" + name.replace("_", "-"), dest=name, type=int, default=None)
     ap.add_argument("--reg-budget", type=int, default=0)
     args = ap.parse_args()
@@ -256,7 +256,7 @@ def main():
     else:
         r = bench_sddmm(args, torch, parpy, W)
     default_cfg = not any(getattr(args, n) is not None for n in ("opt_vectorize", "opt_lds_rows", "opt_reg_cache",
-                                                                 "opt_hoist_invariant", "opt_narrow_index", "opt_unswitch", "opt_gather_transpose", "opt_nontemporal", "opt_mfma_sddmm"))
+                                                                 "opt_hoist_invariant", "opt_narrow_index", "opt_unswitch", "opt_gather_transpose", "opt_nontemporal", "opt_noalias_scopes", "opt_mfma_sddmm"))
     if default_cfg and not args.reg_budget:
         r["roofline"]["traffic"] = _profiled_traffic(args.workload)
     r.update({"n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "scaling": "weak", "vs_baseline": None,

@@ -153,9 +153,6 @@ def get_string_wrapper(kernel_name, key, grid, block, opts):
     g = (ctypes.c_int64 * 3)(*grid)
     b = (ctypes.c_int64 * 3)(*block)
 
-    if opts.use_cuda_graphs:
-        lib.parpy_hip_plan_set_graph(plan, 1)
-
     def wrapper(*args):
         flat = [x for a in args for x in _expand_arg(a)]
         storage = []

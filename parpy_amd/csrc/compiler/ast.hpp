@@ -242,7 +242,7 @@ struct Stmt {
     Alloc,      // id = device allocation of iv elements of type ty.sz
     Free,       // free id
     Launch,     // kernel launch: fname, grid/block, args
-    Scope,      // { body }
+    Scope,      // { body }; with args: the pointer variables in args do not alias each other inside
     WaveReduce, // id = wave_reduce<bop>(id)
     LdsDecl,    // __shared__ ty.sz id[iv]
     RegDecl,    // ty.sz id[iv] (per-thread register array)
@@ -363,6 +363,7 @@ struct Options {  // src/option.rs:14-108
   bool opt_mfma_sddmm = false;  // per-thread dot products on the matrix cores (4x4x1 tiles): measured slower, opt-in
   bool opt_unswitch = false;   // measured slower on the HMM kernels (higher register pressure): opt-in
   bool opt_gather_transpose = true;
+  bool opt_noalias_scopes = false; // aliases that always name different arrays are declared not to alias; measured slower on the HMM kernels: opt-in
   bool opt_nontemporal = true;   // non-temporal stores to arrays a kernel only writes
   int64_t reg_budget = 0;     // 32-bit registers per thread the caching passes may claim (0 = by block size)
   bool assume_aligned = true;  // array arguments are at least 16-byte aligned

@@ -947,6 +947,116 @@ struct Pass {
     k.body = {nr};
   }
 
+  // ================================================================ no-alias scopes for array aliases
+  // `src = a; dst = b; if (c) { src = b; dst = a; } <rest>`: in <rest> the two aliases always name
+  // different arrays, but the target compiler only sees two selected pointers that may be equal, so
+  // it keeps every load from `src` behind the preceding store to `dst`.  When every combination of
+  // the selections gives pairwise different arrays, and <rest> reaches those arrays through the
+  // aliases only, <rest> is put into a scope whose parameters are the aliases, declared not to
+  // alias each other.  Loads of the (independent) iterations that a thread runs of a parallel loop
+  // can then be shared and merged: the four states of a thread that have the same predecessors load
+  // them once, and own-state loads and stores become 128-bit LDS accesses.
+  static bool is_alias_type(const Type& t) { return t.k == Type::Pointer || (t.k == Type::Tensor && !t.shape.empty()); }
+
+  using AliasCfg = std::map<Name, Name>;
+
+  static bool alias_target(const E& e, const AliasCfg& cfg, Name* out) {
+    if (!e || e->k != Expr::Var) return false;
+    auto it = cfg.find(e->name);
+    *out = it == cfg.end() ? e->name : it->second;
+    return true;
+  }
+
+  // statements that only (re)point aliases: applies them to every configuration, false if anything else is found
+  static bool apply_alias_stmt(const S& st, std::vector<AliasCfg>& cfgs, std::vector<Name>& order) {
+    if ((st->k == Stmt::Def && is_alias_type(st->ty)) ||
+        (st->k == Stmt::Assign && st->dst->k == Expr::Var && is_alias_type(st->dst->ty))) {
+      Name a = st->k == Stmt::Def ? st->id : st->dst->name;
+      for (auto& c : cfgs) {
+        Name t;
+        if (!alias_target(st->expr, c, &t)) return false;
+        c[a] = t;
+      }
+      if (std::find(order.begin(), order.end(), a) == order.end()) order.push_back(a);
+      return true;
+    }
+    if (st->k == Stmt::If && !(st->body.empty() && st->els.empty())) {
+      std::vector<AliasCfg> then_c = cfgs, else_c = cfgs;
+      for (auto& c : st->body) if (!apply_alias_stmt(c, then_c, order)) return false;
+      for (auto& c : st->els) if (!apply_alias_stmt(c, else_c, order)) return false;
+      cfgs = then_c;
+      cfgs.insert(cfgs.end(), else_c.begin(), else_c.end());
+      return cfgs.size() <= 16;
+    }
+    return false;
+  }
+
+  Stmts noalias_scopes(const Stmts& ss) {
+    Stmts cur;
+    for (auto& s : ss) {
+      auto r = clone(s);
+      r->body = noalias_scopes(s->body);
+      r->els = noalias_scopes(s->els);
+      cur.push_back(r);
+    }
+    // the first run of alias-only statements of this block
+    size_t a = 0;
+    while (a < cur.size() && !(cur[a]->k == Stmt::Def && is_alias_type(cur[a]->ty))) ++a;
+    if (a == cur.size()) return cur;
+    std::vector<AliasCfg> cfgs(1);
+    std::vector<Name> order;
+    size_t b = a;
+    while (b < cur.size()) {
+      std::vector<AliasCfg> trial = cfgs;
+      std::vector<Name> otrial = order;
+      if (!apply_alias_stmt(cur[b], trial, otrial)) break;
+      cfgs = trial;
+      order = otrial;
+      ++b;
+    }
+    if (order.size() < 2 || b == cur.size()) return cur;
+    std::set<Name> targets;
+    for (auto& c : cfgs) {
+      std::set<Name> seen;
+      for (auto& n : order) {
+        auto it = c.find(n);
+        if (it == c.end() || !seen.insert(it->second).second) return cur;  // two aliases may name one array
+        targets.insert(it->second);
+      }
+    }
+    // the rest of the block must reach the arrays through the aliases only and leave the aliases alone
+    bool clean = true;
+    std::map<Name, Type> types;
+    Stmts rest(cur.begin() + b, cur.end());
+    visit_stmts(rest, [&](const S& st) {
+      if (st->k == Stmt::Def && (targets.count(st->id) || std::count(order.begin(), order.end(), st->id))) clean = false;
+      if (st->k == Stmt::Assign && st->dst->k == Expr::Var && std::count(order.begin(), order.end(), st->dst->name)) clean = false;
+      if ((st->k == Stmt::Def || (st->k == Stmt::Assign && st->dst->k == Expr::Var)) && is_alias_type(st->k == Stmt::Def ? st->ty : st->dst->ty))
+        clean = false;  // a further alias inside the scope could name the same arrays
+      auto scan = [&](const E& e) {
+        visit_exprs(e, [&](const E& x) {
+          if (x->k != Expr::Var) return;
+          if (targets.count(x->name)) clean = false;
+          if (std::count(order.begin(), order.end(), x->name)) types[x->name] = x->ty;
+        });
+      };
+      scan(st->dst); scan(st->expr); scan(st->lo); scan(st->hi);
+      for (auto& e : st->args) scan(e);
+    });
+    if (!clean) return cur;
+    std::vector<E> params;
+    for (auto& n : order)
+      if (types.count(n) && types[n].k == Type::Pointer) params.push_back(mk_var(n, types[n]));
+    if (params.size() < 2) return cur;
+    auto scope = std::make_shared<Stmt>();
+    scope->k = Stmt::Scope;
+    scope->args = params;
+    scope->body = rest;
+    Stmts out(cur.begin(), cur.begin() + b);
+    out.push_back(scope);
+    return out;
+  }
+
   // ================================================================ dot products on the matrix cores
   // `t = t + X[..] * Y[..]` in an innermost sequential f32 loop of constant length is a dot
   // product that every thread computes for itself.  v_mfma_f32_4x4x1 multiplies, for each group
@@ -1231,6 +1341,7 @@ void hip_optimize(Program& p, const Options& opts, NameGen& gen) {
     int64_t budget = pass.reg_budget();
     if (opts.opt_hoist_invariant) k.body = pass.hoist_invariant(k.body, &budget, false);
     if (opts.opt_reg_cache) pass.reg_cache(&budget);
+    if (opts.opt_noalias_scopes) k.body = pass.noalias_scopes(k.body);
     pass.mark_read_only();
     k.aligned_params = opts.assume_aligned;
   }

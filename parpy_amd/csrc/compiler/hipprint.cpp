@@ -558,6 +558,19 @@ struct DevicePrinter {
         break;
       case Stmt::Sync: os << ind(n) << "__syncthreads();\n"; break;
       case Stmt::Scope:
+        if (!s->args.empty()) {
+          // an immediately invoked, always inlined lambda: its restrict-qualified parameters shadow
+          // the pointer variables of the same names, which is how the no-alias fact reaches the optimiser
+          std::string params, actuals;
+          for (size_t a = 0; a < s->args.size(); ++a) {
+            params += (a ? ", " : "") + ctype(s->args[a]->ty) + " __restrict__ " + s->args[a]->name.str();
+            actuals += (a ? ", " : "") + s->args[a]->name.str();
+          }
+          os << ind(n) << "[&](" << params << ") __attribute__((always_inline)) {\n";
+          pstmts(s->body, n + 2);
+          os << ind(n) << "}(" << actuals << ");\n";
+          break;
+        }
         os << ind(n) << "{\n";
         pstmts(s->body, n + 2);
         os << ind(n) << "}\n";

@@ -138,3 +138,17 @@ def column_sums(x, out, N, M):
         for i in range(N):
             acc = acc + x[i, j]
         out[j] = acc
+
+
+def alias_maybe_same(a, b, N, M, steps):
+    """Two aliases of which one may end up naming the same array as the other."""
+    parpy.label('N')
+    for i in range(N):
+        for t in range(steps):
+            src = a
+            dst = b
+            if t & 1:
+                dst = a
+            parpy.label('M')
+            for j in range(M):
+                dst[i, j] = src[i, j] + float32(1.0)

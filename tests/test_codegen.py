@@ -147,6 +147,23 @@ def test_hmm_single_block_is_one_kernel_with_lds_rows():
     assert "lds_alpha" not in s0 and "inv_hmm" not in s0
 
 
+def test_noalias_scope_wraps_the_step_body_when_aliases_never_coincide():
+    hmm, seqs, args = _hmm_args(4)
+    o = opts_for({'inst': parpy.threads(4), 'state': parpy.threads(256)}, opt_noalias_scopes=True)
+    s = compiles(parpy.print_compiled(W.forward_syn, args, o))
+    assert re.search(r"\[&\]\(__attribute__\(\(address_space\(3\)\)\) float\* __restrict__ alpha_src_\d+, "
+                     r"__attribute__\(\(address_space\(3\)\)\) float\* __restrict__ alpha_dst_\d+\) __attribute__\(\(always_inline\)\) \{", s)
+    assert "__restrict__ alpha_src" not in compiles(parpy.print_compiled(W.forward_syn, args, opts_for({'inst': parpy.threads(4), 'state': parpy.threads(256)})))
+    # two aliases that may name the same array: no scope
+    x = np.zeros((4, 64), dtype=np.float32)
+    s = compiles(parpy.print_compiled(K.alias_maybe_same, [x, x.copy(), 4, 64, 3], o_for_alias()))
+    assert not re.search(r"__restrict__ (src|dst)_\d", s)
+
+
+def o_for_alias():
+    return opts_for({'N': parpy.threads(4), 'M': parpy.threads(64)}, opt_noalias_scopes=True)
+
+
 def test_hmm_multi_block_hoists_time_loop_to_host():
     hmm, seqs, args = _hmm_args(5, maxlen=20)
     s = compiles(parpy.print_compiled(W.forward_syn, args, opts_for({'inst': parpy.threads(4), 'state': parpy.threads(2048).tpb(512)})))

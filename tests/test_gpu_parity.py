@@ -177,7 +177,7 @@ def test_forward_synthetic_vs_oracle(k, threads):
 
 @pytest.mark.parametrize("flags", [
     {"opt_lds_rows": False}, {"opt_vectorize": False}, {"opt_hoist_invariant": False}, {"opt_narrow_index": False},
-    {"opt_unswitch": True}, {"opt_lds_rows": False, "opt_vectorize": False, "opt_hoist_invariant": False},
+    {"opt_unswitch": True}, {"opt_noalias_scopes": True}, {"opt_lds_rows": False, "opt_vectorize": False, "opt_hoist_invariant": False},
 ], ids=lambda f: ",".join(f"{k}={int(v)}" for k, v in f.items()))
 def test_forward_synthetic_each_memory_pass_preserves_results(flags):
     hmm, seqs = W.synthetic_hmm(5, n_inst=8, min_len=50, max_len=200)
@@ -365,3 +365,18 @@ def test_graph_replay_of_host_hoisted_time_loop():
     from parpy_amd import _fun_cache
     replays = [w.graph_replays() for w in _fun_cache.values() if w.__name__ == "forward_syn"]
     assert max(replays) >= 6 and max(w.launch_count() for w in _fun_cache.values() if w.__name__ == "forward_syn") >= 119
+
+
+@pytest.mark.parametrize("noalias", [False, True])
+def test_aliases_that_may_coincide(noalias):
+    rng = np.random.default_rng(3)
+    a, b = rng.standard_normal((4, 64)).astype(np.float32), rng.standard_normal((4, 64)).astype(np.float32)
+    wa, wb = a.copy(), b.copy()
+    for t in range(3):
+        if t & 1:
+            wa = wa + np.float32(1.0)
+        else:
+            wb = wa + np.float32(1.0)
+    ad, bd = torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda()
+    parpy.jit(K.alias_maybe_same)(ad, bd, 4, 64, 3, opts=opts_for({'N': parpy.threads(4), 'M': parpy.threads(64)}, opt_noalias_scopes=noalias))
+    assert np.array_equal(ad.cpu().numpy(), wa) and np.array_equal(bd.cpu().numpy(), wb)
