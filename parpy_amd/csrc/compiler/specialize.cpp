@@ -360,6 +360,70 @@ struct SliceExpander {
     return f;
   }
 
+  // Shapes of slice statements are checked before they are expanded, the way the reference
+  // type-checks shapes first (src/py/type_check.rs:235-270 unification with broadcasting from
+  // the right, :720-738 rank of a subscript).
+  static std::string shape_str(const std::vector<int64_t>& s, const char* sep) {
+    std::string r;
+    for (size_t k = 0; k < s.size(); ++k) r += (k ? sep : "") + std::to_string(s[k]);
+    return r;
+  }
+
+  std::vector<int64_t> unify(const std::vector<int64_t>& l, const std::vector<int64_t>& r, const Info& i) {
+    std::vector<int64_t> acc;
+    size_t n = std::max(l.size(), r.size());
+    for (size_t k = 0; k < n; ++k) {
+      bool hl = k < l.size(), hr = k < r.size();
+      int64_t a = hl ? l[l.size() - 1 - k] : 0, b = hr ? r[r.size() - 1 - k] : 0;
+      if (hl && hr && !(a == b || a == 1 || b == 1))
+        fail_ty(i, "Found incompatible shapes " + shape_str(l, ", ") + " and " + shape_str(r, ", "));
+      acc.push_back(hl ? a : b);
+    }
+    std::reverse(acc.begin(), acc.end());
+    return acc;
+  }
+
+  std::vector<int64_t> shape_of(const E& e) {
+    if (!e) return {};
+    switch (e->k) {
+      case Expr::Var: {
+        auto it = arrays.find(e->name);
+        return it != arrays.end() && it->second.is_array() ? it->second.shape : std::vector<int64_t>{};
+      }
+      case Expr::Subscript: {
+        if (e->args[0]->k != Expr::Var) fail_rt(e->i, "Target of slice must be a variable.");
+        auto it = arrays.find(e->args[0]->name);
+        if (it == arrays.end() || !it->second.is_array()) return {};
+        const auto& full = it->second.shape;
+        auto idxs = index_list(e->args[1]);
+        if (idxs.size() > full.size())
+          fail_ty(e->i, "Indexing with " + std::to_string(idxs.size()) + " dimensions on tensor of shape [" + shape_str(full, ",") + "]");
+        std::vector<int64_t> r;
+        if (count_slices_idx(e->args[1]) > 0 && idxs.size() == full.size()) r = slice_shape(e);
+        for (size_t d = idxs.size(); d < full.size(); ++d) r.push_back(full[d]);
+        return r;
+      }
+      case Expr::BinOpE: return unify(shape_of(e->args[0]), shape_of(e->args[1]), e->i);
+      case Expr::IfExpr: return unify(shape_of(e->args[1]), shape_of(e->args[2]), e->i);
+      case Expr::BuiltinE: {
+        BinOp op;
+        if (reduction_builtin(e, &op)) {
+          auto s = shape_of(e->args[0]);
+          if (!e->has_axis) return {};
+          int64_t n = (int64_t)s.size(), ax = e->iv;
+          if (n == 0 || ax >= n || ax < -n) return s;   // reported with the slice counts below
+          s.erase(s.begin() + (size_t)(((ax % n) + n) % n));
+          return s;
+        }
+        std::vector<int64_t> r;
+        for (auto& a : e->args) r = unify(r, shape_of(a), e->i);
+        return r;
+      }
+      case Expr::UnOpE: case Expr::Convert: return shape_of(e->args[0]);
+      default: return {};
+    }
+  }
+
   // src/py/slices.rs:362-486
   S expand_assignment(const S& s) {
     bool is_def = s->k == Stmt::Def;
@@ -370,6 +434,10 @@ struct SliceExpander {
     int nslices = std::max(lslices, rslices);
     if (nslices == 0) return s;
     const Info& i = s->i;
+    {
+      auto rs = shape_of(rhs);
+      if (!is_def) unify(shape_of(lhs), rs, i);
+    }
     std::vector<std::string> labels = s->labels;
 
     BinOp op = BinOp::Add;
@@ -381,6 +449,9 @@ struct SliceExpander {
     std::vector<int64_t> shape;
     bool found = false;
     if (!is_reduce) {
+      if (lslices < rslices)
+        fail_rt(i, "Slice statements cannot have more slice dimensions in the right-hand side expression than in "
+                   "the left-hand side expression.");
       if (is_def) fail_rt(i, "Slice expression cannot be assigned to fresh variable " + s->id.s + ".");
       collect_shape(lhs, shape, found);
     } else {
