@@ -186,8 +186,32 @@ def time_call(fun, *args, opts):
 
 
 def external(ext_name, backend, target, header=None, parallelize=LoopPar()):
-    """Declare an externally defined device function (not available in the HIP backend yet)."""
-    raise RuntimeError("External functions are not supported by the HIP backend yet")
+    """Declare that the decorated function stands for the device function `ext_name`, defined in
+    `header` (found through `opts.includes`) -- python/parpy/__init__.py:201-223 of the reference.
+
+    The decorated Python function is what runs when it is called outside jitted code; inside
+    jitted code a call compiles to a call of `ext_name`.  Parameters and result carry type
+    annotations from `parpy.types` (scalars, or `types.pointer(sz)` for array arguments).
+    """
+    import inspect
+    globs = inspect.currentframe().f_back.f_globals
+    locs = inspect.currentframe().f_back.f_locals
+
+    def external_wrap(fn):
+        import functools
+
+        @functools.wraps(fn)
+        def inner(*args):
+            return fn(*args)
+        if target != Target.Device:
+            raise RuntimeError(f"Host externals are not supported in the {backend} backend")
+        if not isinstance(parallelize, LoopPar):
+            raise RuntimeError("The parallelize argument of an external must be a LoopPar")
+        ext_decl = compiler.declare_external(fn, ext_name, backend, header, parallelize, (globs, locs))
+        _ext_decls.setdefault(backend, {})[fn.__name__] = ext_decl
+        _ext_tops[fn.__name__] = ext_decl
+        return inner
+    return external_wrap
 
 
 def jit(fun):

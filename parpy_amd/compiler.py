@@ -113,6 +113,30 @@ def python_to_ir(tree, info, tops, vars):
     return IrAst(out.value, info[0])
 
 
+def declare_external(fn, ext_name, backend, header, parallelize, vars):
+    """Parsed declaration of an external device function (the reference's parpy.declare_external)."""
+    import ast as pyast
+    import inspect
+    import textwrap
+    lib = _load()
+    src, first = inspect.getsourcelines(fn)
+    tree = pyast.parse(textwrap.dedent("".join(src)))
+    filepath = inspect.getfile(fn)
+    try:
+        text = frontend.external_to_sexpr(tree, (filepath, first - 1, 0), vars, ext_name, header,
+                                          {CompileBackend.Auto: 0, CompileBackend.Cuda: 1, CompileBackend.Metal: 2,
+                                           CompileBackend.Hip: 3}[backend], parallelize.nthreads)
+    except frontend.FrontendError as e:
+        raise RuntimeError(str(e)) from None
+    out = ctypes.c_void_p()
+    cnames = (ctypes.c_char_p * 1)()
+    chandles = (ctypes.c_void_p * 1)()
+    rc = lib.parpy_hipc_parse(text.encode("utf-8"), cnames, chandles, 0, ctypes.byref(out))
+    if rc != 0:
+        _raise_last_error(lib, filepath)
+    return IrAst(out.value, filepath)
+
+
 def get_function_name(ir_ast):
     return _load().parpy_hipc_fun_name(ir_ast.handle).decode()
 

@@ -128,6 +128,16 @@ struct NameGen {
 struct Expr;
 using E = std::shared_ptr<const Expr>;
 
+// Signature of an externally defined device function (parpy.external): what a call site needs to
+// type its arguments and what the printer needs to emit the call and the include.
+struct ExtSig {
+  std::string py_name, name, header;
+  std::vector<Type> params;
+  Type ret;
+  int backend = 3;          // Backend the declaration was made for (as the enum's integer value)
+  int64_t par_threads = 0;  // > 0: the function is executed by that many threads of a workgroup together
+};
+
 struct Expr {
   enum Kind {
     Var, Int, Float, Bool, Str, UnOpE, BinOpE, IfExpr, Subscript, Slice, Tuple, BuiltinE, Call,
@@ -156,6 +166,7 @@ struct Expr {
   // the HIP memory passes).
   std::vector<E> dim_idx;
   std::vector<int64_t> dim_shape;
+  std::shared_ptr<const ExtSig> ext;  // Call only: the external the call refers to
 };
 
 E mk_var(const Name& n, const Type& ty, const Info& i = Info());
@@ -337,6 +348,7 @@ struct FunDef {
 
 // Function as parsed at decoration time: untyped, labels attached, callees inlined.
 struct ParsedFun {
+  std::shared_ptr<const ExtSig> ext;  // set for an external declaration (fun then only carries the name)
   FunDef fun;
   NameGen gen;
   std::string source_text;  // printable form, used for cache keys

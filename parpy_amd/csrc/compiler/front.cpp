@@ -356,7 +356,68 @@ struct Inliner {
       }
       return e;
     }
-    return map_children(e, [&](const E& c) { return sub_expr(c, sub); });
+    E r = map_children(e, [&](const E& c) { return sub_expr(c, sub); });
+    return merge_subscripts(r);
+  }
+
+  // A parameter bound to a partially indexed array (`f(x[i])`) turns the callee's `x[j]` into
+  // `x[i][j]`: one subscript with the indices in sequence.
+  static E merge_subscripts(const E& e) {
+    if (e->k != Expr::Subscript || e->args[0]->k != Expr::Subscript) return e;
+    const E& inner = e->args[0];
+    auto list = [](const E& idx) { return idx->k == Expr::Tuple ? idx->args : std::vector<E>{idx}; };
+    std::vector<E> idxs = list(inner->args[1]);
+    for (auto& x : idxs)
+      if (x->k == Expr::Slice) return e;  // a slice of a slice is left for the slice pass to reject
+    for (auto& x : list(e->args[1])) idxs.push_back(x);
+    auto t = std::make_shared<Expr>();
+    t->k = Expr::Tuple;
+    t->args = idxs;
+    t->i = e->args[1]->i;
+    auto r = std::make_shared<Expr>(*e);
+    r->args = {inner->args[0], E(t)};
+    return merge_subscripts(r);
+  }
+
+  // Calls inside expressions.  A call of an external stays a call (its signature is attached); a
+  // call of a jitted function is replaced by the value it returns, with the statements in front
+  // of its final `return` placed before the statement that contains the call.
+  E inline_expr(const E& e, Stmts& pre) {
+    if (!e) return e;
+    E r = map_children(e, [&](const E& c) { return inline_expr(c, pre); });
+    if (r->k != Expr::Call) return r;
+    auto it = tops.find(r->sval);
+    if (it == tops.end()) fail_rt(r->i, "Call to unknown function " + r->sval);
+    const ParsedFun* pf = it->second;
+    if (pf->ext) {
+      auto c = std::make_shared<Expr>(*r);
+      c->ext = pf->ext;
+      return c;
+    }
+    const FunDef& f = pf->fun;
+    if (f.params.size() != r->args.size())
+      fail_rt(r->i, "Function " + f.id.s + " expected " + std::to_string(f.params.size()) + " arguments, but received " +
+                        std::to_string(r->args.size()) + ".");
+    if (f.body.empty() || f.body.back()->k != Stmt::Return)
+      fail_ty(r->i, "Unknown return type of function " + f.id.s);
+    Sub sub;
+    for (size_t k = 0; k < f.params.size(); ++k) {
+      E a = r->args[k];
+      if (f.params[k].ty.k == Type::Tensor && f.params[k].ty.shape.empty()) {
+        // an annotated scalar parameter: the argument is converted to the declared type
+        auto c = std::make_shared<Expr>();
+        c->k = Expr::BuiltinE;
+        c->fn = Builtin::Convert;
+        c->ty = Type::scalar(f.params[k].ty.sz);
+        c->args = {a};
+        c->i = a->i;
+        a = c;
+      }
+      sub.params[f.params[k].id] = a;
+    }
+    Stmts head(f.body.begin(), f.body.end() - 1);
+    for (auto& st : sub_stmts(head, sub)) pre.push_back(st);
+    return sub_expr(f.body.back()->expr, sub);
   }
 
   Stmts sub_stmts(const Stmts& ss, Sub& sub) {
@@ -395,17 +456,22 @@ struct Inliner {
         if (f.params.size() != s->args.size())
           fail_rt(f.i, "Function " + f.id.s + " expected " + std::to_string(f.params.size()) +
                            " arguments, but received " + std::to_string(s->args.size()) + ".");
+        if (it->second->ext) fail_rt(s->i, "Cannot inline call to external function " + s->fname);
         Sub sub;
-        for (size_t k = 0; k < f.params.size(); ++k) sub.params[f.params[k].id] = s->args[k];
+        for (size_t k = 0; k < f.params.size(); ++k) sub.params[f.params[k].id] = inline_expr(s->args[k], out);
         Stmts body = sub_stmts(f.body, sub);
         for (auto& b : body) out.push_back(b);
         continue;
       }
-      if (s->body.empty() && s->els.empty()) {
-        out.push_back(s);
-        continue;
-      }
       auto r = std::make_shared<Stmt>(*s);
+      Stmts pre;
+      if (r->dst) r->dst = inline_expr(r->dst, pre);
+      if (r->expr) r->expr = inline_expr(r->expr, pre);
+      if (r->lo) r->lo = inline_expr(r->lo, pre);
+      if (r->hi) r->hi = inline_expr(r->hi, pre);
+      if (!pre.empty() && s->k == Stmt::While)
+        fail_rt(s->i, "A function called in the condition of a while loop must consist of a single return statement");
+      for (auto& q : pre) out.push_back(q);
       r->body = run(s->body);
       r->els = run(s->els);
       out.push_back(r);
@@ -421,6 +487,30 @@ std::unique_ptr<ParsedFun> parse_function(const std::string& sexpr,
   SXP x = parse_sexpr(sexpr);
   auto pf = std::make_unique<ParsedFun>();
   Reader rd;
+  if (x->head() == "ext") {
+    // (ext "python name" "target name" <return annotation> (params (p name annotation info)...) "header" backend nthreads info)
+    auto sig = std::make_shared<ExtSig>();
+    sig->py_name = x->at(1)->atom;
+    sig->name = x->at(2)->atom;
+    Info i = parse_info(x->at(8));
+    if (x->at(3)->is_sym("none")) fail_rt(i, "Unsupported return type annotation on external function");
+    sig->ret = rd.annotation(x->at(3), i);
+    if (!sig->ret.is_scalar()) fail_rt(i, "Unsupported return type annotation on external function");
+    const SXP& ps = x->at(4);
+    for (size_t k = 1; k < ps->size(); ++k) {
+      Info pi = parse_info(ps->at(k)->at(3));
+      if (ps->at(k)->at(2)->is_sym("none")) fail_rt(pi, "Unsupported parameter type annotation");
+      sig->params.push_back(rd.annotation(ps->at(k)->at(2), pi));
+    }
+    sig->header = x->at(5)->atom;
+    sig->backend = (int)x->at(6)->as_int();
+    sig->par_threads = x->at(7)->as_int();
+    pf->fun.id = Name{sig->py_name, 0};
+    pf->fun.i = i;
+    pf->ext = sig;
+    pf->source_text = "external " + sig->py_name + " = " + sig->name;
+    return pf;
+  }
   pf->fun = rd.fun(x);
 
   // symbolize: parameters first, then the body

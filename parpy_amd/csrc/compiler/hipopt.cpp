@@ -1130,6 +1130,15 @@ struct Pass {
         if (s->k == Stmt::Assign && s->dst->k == Expr::Var && (s->dst->ty.is_array() || s->dst->ty.is_pointer()))
           bases(s->expr, alias_of[s->dst->name]);
         if (s->k == Stmt::Assign && s->dst->k == Expr::Index) bases(s->dst->args[0], written);
+        // an array handed to an external device function may be written by it
+        auto calls = [&](const E& root) {
+          visit_exprs(root, [&](const E& x) {
+            if (x->k != Expr::Call || !x->ext) return;
+            for (auto& a : x->args)
+              if (a->k == Expr::AddrOf || (a->k == Expr::Var && !a->ty.is_scalar())) bases(a, written);
+          });
+        };
+        calls(s->expr); calls(s->dst); calls(s->lo); calls(s->hi);
       });
     }
     for (auto& p : k.params) p.read_only = p.ty.is_pointer() && !written.count(p.id);

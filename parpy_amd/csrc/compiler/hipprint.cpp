@@ -386,7 +386,7 @@ struct DevicePrinter {
       case Expr::RegElem: return e->name.str() + "[" + pexpr(e->args[0]) + "]";
       case Expr::Raw: return e->sval;
       case Expr::Call: {
-        std::string out = e->sval + "(";
+        std::string out = (e->ext ? e->ext->name : e->sval) + "(";
         for (size_t a = 0; a < e->args.size(); ++a) out += (a ? ", " : "") + pexpr(e->args[a]);
         return out + ")";
       }
@@ -814,6 +814,17 @@ std::string hip_print_device(const Program& p, const Options& opts) {
   std::ostringstream out;
   out << PREAMBLE;
   for (auto& inc : p.includes) out << "#include \"" << inc << "\"\n";
+  // headers of the external device functions the kernels call (written as given: <x.h> or "x.h")
+  std::set<std::string> headers;
+  for (auto& k : p.kernels)
+    visit_stmts(k.body, [&](const S& st) {
+      auto scan = [&](const E& e) {
+        visit_exprs(e, [&](const E& x) { if (x->k == Expr::Call && x->ext && !x->ext->header.empty()) headers.insert(x->ext->header); });
+      };
+      scan(st->dst); scan(st->expr); scan(st->lo); scan(st->hi);
+      for (auto& a : st->args) scan(a);
+    });
+  for (auto& h : headers) out << "#include " << ((h[0] == '<' || h[0] == '"') ? h : "\"" + h + "\"") << "\n";
   for (auto& d : p.preamble) out << d << "\n";
   DevicePrinter dp(opts);
   for (auto& k : p.kernels) out << "\n" << dp.kernel_text(k);

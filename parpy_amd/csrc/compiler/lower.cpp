@@ -6,6 +6,8 @@
 // Counterpart of the reference's src/ir/from_py_ast.rs:176-214,283-297
 // (indexing), :342-386 (labels -> LoopPar), :402-413 (GPU context) and
 // src/ir/eliminate_gpu_context.rs:5-30.
+#include <functional>
+
 #include "passes.hpp"
 
 namespace parpy {
@@ -58,6 +60,40 @@ struct Lowerer {
     return map_children(e, [&](const E& c) { return lower_expr(c); });
   }
 
+  // An external declared with `parallelize=threads(n)` is executed by n threads of a workgroup
+  // together (it indexes its data with threadIdx.x itself).  The statement that calls it becomes
+  // a parallel layer of n threads, every one of which makes the call (src/gpu/par.rs:88-103);
+  // the value is then stored by the statement proper, which the store-hazard pass limits to one thread.
+  int64_t parallel_external_threads(const S& s) {
+    if (s->k != Stmt::Assign && s->k != Stmt::Def) return 0;
+    int64_t n = 0;
+    visit_exprs(s->expr, [&](const E& x) {
+      if (x->k != Expr::Call || !x->ext || x->ext->par_threads <= 0) return;
+      if (n != 0 && n != x->ext->par_threads) fail_rt(s->i, "Found calls of externals with different numbers of threads in one statement");
+      n = x->ext->par_threads;
+    });
+    return n;
+  }
+
+  S cooperative_call(const S& s, int64_t n) {
+    if (s->k == Stmt::Def) fail_rt(s->i, "The result of an external that runs on several threads must be assigned to an array element");
+    Stmts body;
+    std::function<E(const E&)> pull = [&](const E& e) -> E {
+      if (!e) return e;
+      if (e->k == Expr::Call && e->ext && e->ext->par_threads > 0) {
+        Name t = gen.fresh("ext_res");
+        body.push_back(mk_def(t, e->ty, lower_expr(e), e->i));
+        return mk_var(t, e->ty, e->i);
+      }
+      return map_children(e, pull);
+    };
+    E rhs = pull(s->expr);
+    body.push_back(mk_assign(lower_expr(s->dst), lower_expr(rhs), s->i));
+    LoopPar p;
+    p.nthreads = n;
+    return mk_for(gen.fresh("ext_lane"), mk_int(0, opts.int_size()), mk_int(n, opts.int_size()), 1, body, p, s->i);
+  }
+
   LoopPar loop_par(const S& s) {
     LoopPar p;
     for (auto& l : s->labels) {
@@ -87,6 +123,10 @@ struct Lowerer {
           Name v = gen.fresh("_gpu_context");
           out.push_back(mk_for(v, mk_int(0, opts.int_size()), mk_int(1, opts.int_size()), 1, body, p, s->i));
         }
+        continue;
+      }
+      if (int64_t n = parallel_external_threads(s)) {
+        out.push_back(cooperative_call(s, n));
         continue;
       }
       auto r = std::const_pointer_cast<Stmt>(std::static_pointer_cast<const Stmt>(map_exprs(s, [&](const E& e) { return lower_expr(e); })));

@@ -420,6 +420,12 @@ struct SliceExpander {
         return r;
       }
       case Expr::UnOpE: case Expr::Convert: return shape_of(e->args[0]);
+      case Expr::Call: {
+        std::vector<int64_t> r;
+        for (size_t k = 0; k < e->args.size(); ++k)
+          if (!(e->ext && k < e->ext->params.size() && e->ext->params[k].is_pointer())) r = unify(r, shape_of(e->args[k]), e->i);
+        return r;
+      }
       default: return {};
     }
   }
@@ -760,6 +766,45 @@ struct TypeChecker {
     return r;
   }
 
+  // Call of an external device function (src/py/type_check.rs:854-877): scalar arguments are
+  // coerced to the declared types, pointer arguments must be arrays of the declared element type,
+  // and every call of one external must pass arrays of the same shapes.
+  std::map<std::string, std::vector<Type>> ext_arg_types;
+
+  E ext_call(const E& e) {
+    if (!e->ext || e->ext->backend != (int)opts.backend) fail_rt(e->i, "Call to unknown function " + e->sval);
+    const ExtSig& sig = *e->ext;
+    if (sig.params.size() != e->args.size())
+      fail_rt(e->i, "Function " + sig.py_name + " expected " + std::to_string(sig.params.size()) + " arguments, but received " +
+                        std::to_string(e->args.size()) + ".");
+    auto r = std::make_shared<Expr>(*e);
+    std::vector<Type> tys;
+    for (size_t k = 0; k < e->args.size(); ++k) {
+      E a = expr(e->args[k]);
+      if (sig.params[k].is_pointer()) {
+        if (!a->ty.is_array() || a->ty.sz != sig.params[k].sz)
+          fail_ty(a->i, "Found incompatible types in function call:\nargument " + std::to_string(k + 1) + " of " + sig.py_name +
+                            " has type " + a->ty.str() + ", expected an array of " + Type::scalar(sig.params[k].sz).str());
+      } else {
+        if (!a->ty.is_scalar())
+          fail_ty(a->i, "Found incompatible types in function call:\nargument " + std::to_string(k + 1) + " of " + sig.py_name +
+                            " has type " + a->ty.str() + ", expected " + sig.params[k].str());
+        a = ensure_scalar(a, sig.params[k].sz);
+      }
+      tys.push_back(a->ty);
+      r->args[k] = a;
+    }
+    auto seen = ext_arg_types.find(sig.py_name);
+    if (seen == ext_arg_types.end()) ext_arg_types[sig.py_name] = tys;
+    else
+      for (size_t k = 0; k < tys.size(); ++k)
+        if (tys[k] != seen->second[k])
+          fail_ty(e->i, "Found incompatible types in function call:\n" + tys[k].str() + " and " + seen->second[k].str() +
+                            " for argument " + std::to_string(k + 1) + " of " + sig.py_name);
+    r->ty = sig.ret;
+    return r;
+  }
+
   E binop(const E& e) {
     E a = expr(e->args[0]), b = expr(e->args[1]);
     const Info& i = e->i;
@@ -838,7 +883,7 @@ struct TypeChecker {
       case Expr::Slice: fail_rt(e->i, "Slice expressions are only allowed in assignment statements.");
       case Expr::Tuple: fail_ty(e->i, "Tuple expressions are only supported as indices");
       case Expr::BuiltinE: return builtin(e);
-      case Expr::Call: fail_ty(e->i, "Calls to user-defined functions inside expressions are not supported by the HIP backend yet");
+      case Expr::Call: return ext_call(e);
       case Expr::Convert: {
         E a = expr(e->args[0]);
         auto r = std::make_shared<Expr>(*e);

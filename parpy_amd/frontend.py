@@ -327,6 +327,31 @@ class _Converter:
         return f"(fun {_quote(fn.name)} {self.info(fn)} {ret} (params {params}) (body {body}))"
 
 
+def external_to_sexpr(tree, info, vars, ext_name, header, backend_code, nthreads):
+    """Serialise the declaration of an external: only the signature of the decorated function is used."""
+    filepath, line_ofs, col_ofs = info
+    globs, locs = vars
+    c = _Converter(filepath, line_ofs, col_ofs, {}, globs, locs)
+    fn = tree.body[0]
+    if not isinstance(fn, pyast.FunctionDef):
+        raise FrontendError("Expected a function definition")
+    params = []
+    for a in fn.args.args:
+        if a.annotation is None:
+            c.err(a, "Unsupported parameter type annotation")
+        params.append(f"(p {_quote(a.arg)} {c.annotation(a.annotation, a)} {c.info(a)})")
+    if fn.returns is None:
+        c.err(fn, "Unsupported return type annotation on external function")
+    try:
+        ret = c.annotation(fn.returns, fn)
+    except FrontendError:
+        c.err(fn, "Unsupported return type annotation on external function")
+    if not ret.startswith("(scalar"):
+        c.err(fn, "Unsupported return type annotation on external function")
+    return (f"(ext {_quote(fn.name)} {_quote(ext_name)} {ret} (params {' '.join(params)}) {_quote(header or '')} "
+            f"{backend_code} {int(nthreads or 0)} {c.info(fn)})")
+
+
 def to_sexpr(tree, info, tops, vars):
     """Serialise a parsed function definition.  `info` = (file, line_ofs, col_ofs),
     `tops` = names of previously jitted functions / externals, `vars` = (globals, locals)."""

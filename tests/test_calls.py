@@ -1,0 +1,291 @@
+"""Calls between jitted functions and calls of external device functions
+(test/test_call.py, test/test_cuda.py:113-225 of the reference, re-targeted to HIP;
+the external targets live in tests/code/hip_utils.h)."""
+import os
+
+import numpy as np
+import pytest
+
+import parpy_amd as parpy
+import parpy_amd.types as types
+from parpy_amd.compile import hiprtc_compile
+
+HIP = parpy.CompileBackend.Hip
+CODE_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "code")
+
+
+def opts_for(p):
+    o = parpy.par(p)
+    o.backend = HIP
+    o.includes += [CODE_DIR]
+    return o
+
+
+def compiles(s, o=None):
+    hiprtc_compile(s[:s.index("// host side")], o or opts_for({}))
+    return s
+
+
+# ---------------------------------------------------------------- jitted callees
+@parpy.jit
+def add_call(x: types.F32, y: types.F32):
+    return x + y
+
+
+@parpy.jit
+def mul_call(x: types.F32, y: types.F32):
+    return x * y
+
+
+@parpy.jit
+def add_then_mul(x: types.F32, y: types.F32, z: types.F32):
+    return mul_call(add_call(x, y), z)
+
+
+@parpy.jit
+def scaled_square(x: types.F32, s: types.F32):
+    t = x * x
+    u = t * s
+    return u + t
+
+
+@parpy.jit
+def add_direct(x, y, N):
+    parpy.label('N')
+    y[:] = add_call(x[:], y[:])
+
+
+@parpy.jit
+def add_mul_nested(x, y, N):
+    parpy.label('N')
+    y[:] = add_then_mul(x[:], y[:], x[:])
+
+
+@parpy.jit
+def with_locals(x, y, N):
+    parpy.label('N')
+    for i in range(N):
+        y[i] = scaled_square(x[i], 0.5)
+
+
+@parpy.jit
+def add_inplace(x, y, M):
+    parpy.label("1d")
+    y[:] += x[:]
+
+
+@parpy.jit
+def add_2d_inplace(x, y, N, M):
+    parpy.label("2d")
+    for i in range(N):
+        add_inplace(x[i], y[i], M)
+
+
+@parpy.jit
+def add_2d_inplace_x2(x, y, z, w, N, M):
+    parpy.label("2d")
+    for i in range(N):
+        add_inplace(x[i], y[i], M)
+        add_inplace(z[i], w[i], M)
+
+
+@parpy.jit
+def add_3d_inplace(x, y, N, M, K):
+    parpy.label('3d')
+    for i in range(N):
+        add_2d_inplace(x[i], y[i], M, K)
+
+
+# ---------------------------------------------------------------- externals
+@parpy.external("sqrtf", HIP, parpy.Target.Device)
+def sqrt_ext(x: types.F32) -> types.F32:
+    return np.sqrt(x)
+
+
+@parpy.external("clamp", HIP, parpy.Target.Device, header="<hip_utils.h>")
+def clamp(x: types.F32, lo: types.F32, hi: types.F32) -> types.F32:
+    return min(max(x, lo), hi)
+
+
+@parpy.external("sum_row_ext", HIP, parpy.Target.Device, header="<hip_utils.h>")
+def sum_row(x: types.pointer(types.F64), n: types.I64) -> types.F64:
+    return np.sum(x[:n])
+
+
+@parpy.external("wave_sum", HIP, parpy.Target.Device, header="<hip_utils.h>", parallelize=parpy.threads(64))
+def wave_sum_custom(x: types.pointer(types.F32)) -> types.F32:
+    return np.sum(x)
+
+
+@parpy.external("_zero", parpy.CompileBackend.Cuda, parpy.Target.Device)
+def zero_for_cuda() -> types.I32:
+    return 0
+
+
+@parpy.jit
+def ext_sqrt(x, y):
+    with parpy.gpu:
+        y[0] = sqrt_ext(x)
+
+
+@parpy.jit
+def clamp_many(out, x):
+    parpy.label('N')
+    out[:] = clamp(x[:], 0.0, 10.0)
+
+
+@parpy.jit
+def sum_ext_seq(x, y, N, M):
+    parpy.label('N')
+    for i in range(N):
+        y[i] = sum_row(x[i], M)
+
+
+@parpy.jit
+def sum_rows_using_ext(out, x, N):
+    parpy.label('N')
+    for i in range(N):
+        out[i] = wave_sum_custom(x[i])
+
+
+F = np.float32
+
+
+# ---------------------------------------------------------------- code generation (no GPU)
+def test_expression_calls_are_inlined():
+    x = np.zeros(10, dtype=F)
+    s = compiles(parpy.print_compiled(add_direct, [x, x.copy(), 10], opts_for({'N': parpy.threads(10)})))
+    assert "add_call" not in s.split("extern \"C\" __global__")[1]
+    compiles(parpy.print_compiled(add_mul_nested, [x, x.copy(), 10], opts_for({'N': parpy.threads(10)})))
+    compiles(parpy.print_compiled(with_locals, [x, x.copy(), 10], opts_for({'N': parpy.threads(10)})))
+
+
+def test_statement_calls_with_sub_tensors():
+    a2, a3 = np.zeros((10, 15), dtype=F), np.zeros((10, 20, 30), dtype=F)
+    compiles(parpy.print_compiled(add_2d_inplace, [a2, a2.copy(), 10, 15], opts_for({'2d': parpy.threads(10), '1d': parpy.threads(15)})))
+    compiles(parpy.print_compiled(add_3d_inplace, [a3, a3.copy(), 10, 20, 30],
+                                  opts_for({'3d': parpy.threads(10), '2d': parpy.threads(20), '1d': parpy.threads(30)})))
+    z = np.zeros((10, 15), dtype=np.int32)
+    compiles(parpy.print_compiled(add_2d_inplace_x2, [a2, a2.copy(), z, z.copy(), 10, 15],
+                                  opts_for({'2d': parpy.threads(10), '1d': parpy.threads(15)})))
+
+
+def test_unknown_and_recursive_callees_are_rejected():
+    def plain(x, y, M):
+        for i in range(M):
+            y[i] += x[i]
+    with pytest.raises(RuntimeError, match=r".*unknown function plain.*"):
+        @parpy.jit
+        def add_2d(x, y, N, M):
+            parpy.label('N')
+            for i in range(N):
+                plain(x[i], y[i], M)
+    with pytest.raises(RuntimeError, match=r".*unknown function reset.*"):
+        @parpy.jit
+        def reset(x, i):
+            with parpy.gpu:
+                if i > 0:
+                    x[i] = 0.0
+                    reset(x, i - 1)
+
+
+def test_external_declarations_are_validated():
+    assert "sqrt_ext" in parpy._ext_decls[HIP]
+    with pytest.raises(RuntimeError, match="Unsupported parameter type annotation"):
+        @parpy.external("dummy", HIP, parpy.Target.Device)
+        def dummy(x: int) -> types.I32:
+            return x
+    with pytest.raises(RuntimeError, match="Unsupported return type annotation on external function"):
+        @parpy.external("dummy", HIP, parpy.Target.Device)
+        def dummy2(x: types.I32) -> int:
+            return x
+    with pytest.raises(RuntimeError, match="Host externals are not supported"):
+        @parpy.external("dummy", HIP, parpy.Target.Host)
+        def dummy3(x: types.I64) -> types.I64:
+            return x
+
+
+def test_external_calls_compile():
+    s = compiles(parpy.print_compiled(ext_sqrt, [F(2.0), np.zeros(1, dtype=F)], opts_for({})))
+    assert "sqrtf(" in s
+    x = np.zeros(10, dtype=F)
+    o = opts_for({'N': parpy.threads(10)})
+    s = compiles(parpy.print_compiled(clamp_many, [x.copy(), x], o), o)
+    assert "#include <hip_utils.h>" in s and "clamp(x_" in s
+    s = compiles(parpy.print_compiled(sum_ext_seq, [np.zeros((10, 20)), np.zeros(10), 10, 20], o), o)
+    assert "sum_row_ext((&x_" in s and "const double* __restrict__ x_" not in s   # the external may write through its pointer
+    s = compiles(parpy.print_compiled(sum_rows_using_ext, [x.copy(), np.zeros((10, 64), dtype=F), 10], o), o)
+    # one workgroup of 64 threads per row makes the call; one thread stores the result
+    assert "<<<dim3(1, 10, 1), dim3(64, 1, 1)" in s and "threadIdx.x == 0" in s
+
+
+def test_external_misuse_is_rejected():
+    with pytest.raises(RuntimeError, match=r"Call to unknown function zero_for_cuda.*"):
+        @parpy.jit
+        def f(x):
+            with parpy.gpu:
+                x[:] = zero_for_cuda()
+        parpy.print_compiled(f, [np.zeros(10, dtype=np.int32)], opts_for({}))
+    with pytest.raises(TypeError, match="incompatible types"):
+        @parpy.jit
+        def g(out, x, y):
+            with parpy.gpu:
+                out[0] = sum_row(x, 10) + sum_row(y, 20)
+        parpy.print_compiled(g, [np.zeros(1), np.zeros(10), np.zeros(20)], opts_for({}))
+
+    @parpy.external("clamp_non_existent", HIP, parpy.Target.Device, header="<hip_utils.h>")
+    def clamp_missing(x: types.F32, lo: types.F32, hi: types.F32) -> types.F32:
+        return x
+
+    @parpy.jit
+    def h(out, x):
+        parpy.label('N')
+        out[:] = clamp_missing(x[:], 0.0, 10.0)
+    o = opts_for({'N': parpy.threads(10)})
+    s = parpy.print_compiled(h, [np.zeros(10, dtype=F), np.zeros(10, dtype=F)], o)
+    with pytest.raises(RuntimeError, match="Compilation of generated HIP code failed"):
+        compiles(s, o)
+
+
+# ---------------------------------------------------------------- results (GPU)
+@pytest.mark.gpu
+def test_calls_give_the_results_of_the_inlined_code():
+    rng = np.random.default_rng(11)
+    x = rng.standard_normal(10).astype(F)
+    y = np.zeros_like(x)
+    add_direct(x, y, 10, opts=opts_for({'N': parpy.threads(10)}))
+    assert np.array_equal(x, y)
+    y = np.zeros_like(x)
+    add_mul_nested(x, y, 10, opts=opts_for({'N': parpy.threads(10)}))
+    assert np.allclose(x ** 2, y)
+    y = np.zeros_like(x)
+    with_locals(x, y, 10, opts=opts_for({'N': parpy.threads(10)}))
+    assert np.allclose(y, 1.5 * x * x)
+    a, b = rng.standard_normal((10, 15)).astype(F), np.zeros((10, 15), dtype=F)
+    add_2d_inplace(a, b, 10, 15, opts=opts_for({'2d': parpy.threads(10), '1d': parpy.threads(15)}))
+    assert np.array_equal(a, b)
+    z, w = rng.integers(0, 10, (10, 15)).astype(np.int32), np.zeros((10, 15), dtype=np.int32)
+    b[:] = 0
+    add_2d_inplace_x2(a, b, z, w, 10, 15, opts=opts_for({'2d': parpy.threads(10), '1d': parpy.threads(15)}))
+    assert np.array_equal(a, b) and np.array_equal(z, w)
+    a3, b3 = rng.standard_normal((10, 20, 30)).astype(F), np.zeros((10, 20, 30), dtype=F)
+    add_3d_inplace(a3, b3, 10, 20, 30, opts=opts_for({'3d': parpy.threads(10), '2d': parpy.threads(20), '1d': parpy.threads(30)}))
+    assert np.array_equal(a3, b3)
+
+
+@pytest.mark.gpu
+def test_externals_run():
+    rng = np.random.default_rng(12)
+    y = np.zeros(1, dtype=F)
+    ext_sqrt(F(2.0), y, opts=opts_for({}))
+    assert np.allclose(y, np.sqrt(F(2.0)))
+    x = (rng.standard_normal(10) * 10).astype(F)
+    out = np.zeros_like(x)
+    clamp_many(out, x, opts=opts_for({'N': parpy.threads(10)}))
+    assert np.array_equal(out, np.clip(x, 0.0, 10.0))
+    xd, yd = rng.standard_normal((10, 20)), np.zeros(10)
+    sum_ext_seq(xd, yd, 10, 20, opts=opts_for({'N': parpy.threads(10)}))
+    assert np.allclose(yd, xd.sum(axis=1))
+    xf, of = rng.standard_normal((10, 64)).astype(F), np.zeros(10, dtype=F)
+    sum_rows_using_ext(of, xf, 10, opts=opts_for({'N': parpy.threads(10)}))
+    assert np.allclose(of, xf.sum(axis=1), atol=1e-5)

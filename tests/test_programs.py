@@ -1,0 +1,215 @@
+"""Whole programs in the style of the reference's regression tests, compiled for gfx950 (CPU part)
+and run against NumPy (GPU part): symmetric rank-k update with a triangular iteration space
+(test/test_syrk.py), CSR SpMV and SpMM with data-dependent loop bounds (test/test_spmv.py,
+test/test_spmm.py), nested loops with different inner thread counts (test/test_sync.py:57-92),
+a Jacobi stencil on shifted slices and matrix products on slices (test/test_slicing.py)."""
+import numpy as np
+import pytest
+
+import parpy_amd as parpy
+from parpy_amd.compile import hiprtc_compile
+from parpy_amd.operators import exp, float32, sum
+
+HIP = parpy.CompileBackend.Hip
+
+
+def opts_for(p, **kw):
+    o = parpy.par(p)
+    o.backend = HIP
+    for k, v in kw.items():
+        setattr(o, k, v)
+    return o
+
+
+def compiles(s):
+    hiprtc_compile(s[:s.index("// host side")], opts_for({}))
+    return s
+
+
+# ---------------------------------------------------------------- programs
+def syrk(alpha, beta, C, A, N, M):
+    parpy.label('i')
+    for i in range(N):
+        parpy.label('j')
+        for j in range(i + 1):
+            C[i, j] = C[i, j] * beta
+            parpy.label('k')
+            for k in range(M):
+                C[i, j] = C[i, j] + alpha * A[i, k] * A[j, k]
+
+
+def spmv(A, x, y):
+    parpy.label('row')
+    for row in range(A["nrows"]):
+        parpy.label('i')
+        for i in range(A["rows"][row], A["rows"][row + 1]):
+            y[row] += A["values"][i] * x[A["cols"][i]]
+
+
+def spmm(A, B, C):
+    parpy.label('i')
+    for i in range(A["nrows"]):
+        parpy.label('j')
+        for j in range(B["ncols"]):
+            parpy.label('aidx')
+            for aidx in range(A["rows"][i], A["rows"][i + 1]):
+                C[i, j] += A["values"][aidx] * B["values"][A["cols"][aidx], j]
+
+
+def exp_then_sum(x, N, M, out):
+    parpy.label('N')
+    for i in range(N):
+        parpy.label('M')
+        for j in range(M):
+            parpy.label('K_1')
+            x[i, j, :] = exp(x[i, j, :])
+        parpy.label('M')
+        for j in range(M):
+            parpy.label('K_2')
+            out[i, j] = sum(x[i, j, :])
+
+
+def jacobi(nsteps, A, B):
+    for t in range(1, nsteps):
+        parpy.label('N')
+        B[1:-1] = (A[:-2] + A[1:-1] + A[2:]) / 3.0
+        parpy.label('N')
+        A[1:-1] = (B[:-2] + B[1:-1] + B[2:]) / 3.0
+
+
+def matmul_rows(a, b, M, N, c):
+    for i in range(M):
+        parpy.label('N')
+        for j in range(N):
+            parpy.label('K')
+            c[i, j] = sum(a[i, :] * b[:, j])
+
+
+def mul_planes(x, y, out):
+    parpy.label('N')
+    parpy.label('M')
+    out[:, :] = x[:, 0, :] * y[0, :, :]
+
+
+# ---------------------------------------------------------------- inputs
+def syrk_data():
+    M, N = 20, 30
+    C = np.fromfunction(lambda i, j: ((i * j + 2) % N) / M, (N, N), dtype=np.float32).astype(np.float32)
+    A = np.fromfunction(lambda i, j: ((i * j + 2) % N) / N, (N, M), dtype=np.float32).astype(np.float32)
+    return 1.5, 1.2, C, A, N, M
+
+
+def random_csr(n, m, density, seed):
+    rng = np.random.default_rng(seed)
+    nnz = int(n * m * density)
+    flat = np.sort(rng.choice(n * m, size=nnz, replace=False))
+    rows, cols = np.divmod(flat, m)
+    crows = np.zeros(n + 1, dtype=np.int64)
+    np.add.at(crows, rows + 1, 1)
+    crows = np.cumsum(crows)
+    vals = rng.standard_normal(nnz).astype(np.float32)
+    dense = np.zeros((n, m), dtype=np.float32)
+    dense[rows, cols] = vals
+    return {"values": vals, "rows": crows, "cols": cols.astype(np.int64), "nrows": n}, dense
+
+
+SYRK_PAR = [{'i': parpy.threads(30)}, {'i': parpy.threads(30), 'k': parpy.threads(64).reduce()},
+            {'i': parpy.threads(30), 'k': parpy.threads(256).reduce()}, {'i': parpy.threads(30), 'k': parpy.threads(1024).reduce()}]
+SPMV_PAR = [{"row": parpy.threads(256)}, {"row": parpy.threads(256), "i": parpy.threads(128).reduce()}]
+SPMM_PAR = [{"i": parpy.threads(128)}, {"i": parpy.threads(128), "j": parpy.threads(64)},
+            {"i": parpy.threads(128), "j": parpy.threads(64), "aidx": parpy.threads(64).reduce()}]
+NEST_PAR = {'N': parpy.threads(10), 'M': parpy.threads(20), 'K_1': parpy.threads(64), 'K_2': parpy.threads(128)}
+
+
+# ---------------------------------------------------------------- code generation (no GPU)
+@pytest.mark.parametrize("p", SYRK_PAR, ids=lambda p: "+".join(p))
+def test_syrk_compiles(p):
+    compiles(parpy.print_compiled(syrk, list(syrk_data()), opts_for(p)))
+
+
+@pytest.mark.parametrize("p", SPMV_PAR, ids=lambda p: "+".join(p))
+def test_spmv_compiles(p):
+    A, _ = random_csr(256, 4096, 0.01, 1)
+    compiles(parpy.print_compiled(spmv, [A, np.zeros(4096, dtype=np.float32), np.zeros(256, dtype=np.float32)], opts_for(p)))
+
+
+@pytest.mark.parametrize("p", SPMM_PAR, ids=lambda p: "+".join(p))
+def test_spmm_compiles(p):
+    A, _ = random_csr(128, 256, 0.02, 2)
+    B = {"values": np.zeros((256, 64), dtype=np.float32), "ncols": 64}
+    compiles(parpy.print_compiled(spmm, [A, B, np.zeros((128, 64), dtype=np.float32)], opts_for(p)))
+
+
+def test_other_programs_compile():
+    x = np.zeros((10, 20, 30), dtype=np.float32)
+    compiles(parpy.print_compiled(exp_then_sum, [x, 10, 20, np.zeros((10, 20), dtype=np.float32)], opts_for(NEST_PAR)))
+    a = np.zeros(10, dtype=np.float32)
+    s = compiles(parpy.print_compiled(jacobi, [5, a, a.copy()], opts_for({'N': parpy.threads(64)})))
+    host = s[s.index("// host side"):]
+    assert host.count("<<<") == 2 and "for (" in host   # the time loop runs on the host: two launches per step
+    compiles(parpy.print_compiled(matmul_rows, [np.zeros((10, 15), dtype=np.float32), np.zeros((15, 20), dtype=np.float32), 10, 20,
+                                                np.zeros((10, 20), dtype=np.float32)], opts_for({'N': parpy.threads(64), 'K': parpy.threads(64)})))
+    compiles(parpy.print_compiled(mul_planes, [np.zeros((10, 4, 15), dtype=np.float32), np.zeros((5, 10, 15), dtype=np.float32),
+                                               np.zeros((10, 15), dtype=np.float32)], opts_for({'N': parpy.threads(64), 'M': parpy.threads(64)})))
+
+
+# ---------------------------------------------------------------- results (GPU)
+@pytest.mark.gpu
+@pytest.mark.parametrize("p", SYRK_PAR, ids=lambda p: "+".join(p))
+def test_syrk(p):
+    alpha, beta, C, A, N, M = syrk_data()
+    want = C.copy()
+    tri = np.tril(np.ones((N, N), dtype=bool))
+    want[tri] = (C * np.float32(beta) + np.float32(alpha) * (A @ A.T))[tri]
+    got = C.copy()
+    parpy.jit(syrk)(alpha, beta, got, A, N, M, opts=opts_for(p))
+    assert np.allclose(got, want, atol=1e-4, rtol=1e-5)
+    assert np.array_equal(got[~tri], C[~tri])     # the upper triangle is not touched
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("p", SPMV_PAR, ids=lambda p: "+".join(p))
+def test_spmv(p):
+    A, dense = random_csr(256, 4096, 0.01, 1)
+    x = np.random.default_rng(5).standard_normal(4096).astype(np.float32)
+    y = np.zeros(256, dtype=np.float32)
+    parpy.jit(spmv)(A, x, y, opts=opts_for(p))
+    assert np.allclose(y, dense.astype(np.float64) @ x, atol=1e-4)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("p", SPMM_PAR, ids=lambda p: "+".join(p))
+def test_spmm(p):
+    A, dense = random_csr(128, 256, 0.02, 2)
+    Bv = np.random.default_rng(6).standard_normal((256, 64)).astype(np.float32)
+    C = np.zeros((128, 64), dtype=np.float32)
+    parpy.jit(spmm)(A, {"values": Bv, "ncols": 64}, C, opts=opts_for(p))
+    assert np.allclose(C, dense.astype(np.float64) @ Bv, atol=1e-4)
+
+
+@pytest.mark.gpu
+def test_nested_loops_with_different_inner_thread_counts():
+    x = np.random.default_rng(7).standard_normal((10, 20, 30)).astype(np.float32)
+    out = np.zeros((10, 20), dtype=np.float32)
+    xd = x.copy()
+    parpy.jit(exp_then_sum)(xd, 10, 20, out, opts=opts_for(NEST_PAR))
+    assert np.allclose(xd, np.exp(x), atol=1e-5, rtol=1e-5)
+    assert np.allclose(out, np.exp(x.astype(np.float64)).sum(axis=2), atol=1e-4, rtol=1e-5)
+
+
+@pytest.mark.gpu
+def test_stencil_and_products_on_slices():
+    rng = np.random.default_rng(8)
+    A, B = rng.standard_normal(10).astype(np.float32), rng.standard_normal(10).astype(np.float32)
+    wa, wb = A.copy(), B.copy()
+    jacobi(5, wa, wb)                              # the function itself, run by the Python interpreter
+    parpy.jit(jacobi)(5, A, B, opts=opts_for({'N': parpy.threads(64)}))
+    assert np.allclose(A, wa, atol=1e-5) and np.allclose(B, wb, atol=1e-5)
+    a, b = rng.standard_normal((10, 15)).astype(np.float32), rng.standard_normal((15, 20)).astype(np.float32)
+    c = np.zeros((10, 20), dtype=np.float32)
+    parpy.jit(matmul_rows)(a, b, 10, 20, c, opts=opts_for({'N': parpy.threads(64), 'K': parpy.threads(64)}))
+    assert np.allclose(c, a @ b, atol=1e-4)
+    x, y = rng.standard_normal((10, 4, 15)).astype(np.float32), rng.standard_normal((5, 10, 15)).astype(np.float32)
+    out = np.zeros((10, 15), dtype=np.float32)
+    parpy.jit(mul_planes)(x, y, out, opts=opts_for({'N': parpy.threads(64), 'M': parpy.threads(64)}))
+    assert np.array_equal(out, x[:, 0, :] * y[0, :, :])
