@@ -368,7 +368,7 @@ struct Inliner {
     auto list = [](const E& idx) { return idx->k == Expr::Tuple ? idx->args : std::vector<E>{idx}; };
     std::vector<E> idxs = list(inner->args[1]);
     for (auto& x : idxs)
-      if (x->k == Expr::Slice) return e;  // a slice of a slice is left for the slice pass to reject
+      if (x->k == Expr::Slice || x->k == Expr::Str) return e;  // slices of slices are rejected later; d["key"][i] stays a field access
     for (auto& x : list(e->args[1])) idxs.push_back(x);
     auto t = std::make_shared<Expr>();
     t->k = Expr::Tuple;
