@@ -58,6 +58,10 @@ class ElemSize(enum.Enum):
     def is_floating_point(self):
         return self in (ElemSize.F16, ElemSize.F32, ElemSize.F64)
 
+    def size(self):
+        """Width of one element in bytes."""
+        return _NBYTES[self]
+
     def __repr__(self):
         return f"ElemSize.{self.name}"
 
