@@ -1336,10 +1336,145 @@ struct GatherTranspose {
   }
 };
 
+// ================================================================ lane groups for per-thread dot products
+// A grid-wide loop whose every iteration runs a long sequential sum over unit-stride rows
+// (`t += X[a*K + d] * Y[b*K + d]`, d = 0..K) makes each lane walk its own rows: one wavefront load
+// touches 64 different cache lines and uses 16 bytes of each, and the line is fetched again for
+// each of the following iterations unless it survives in L1.  Here G = 8 adjacent lanes share one
+// iteration instead: lane g takes the g-th 16-byte piece of every 128-byte line, so each line is
+// requested once, and the eight partial sums are added with three DPP steps.  The launch grows by
+// G; statements after the sum that store to memory are executed by lane 0 of each group.
+struct LaneSplit {
+  Program& p;
+  const Options& opts;
+  NameGen& gen;
+  ElemSize isz;
+  static constexpr int64_t G = 8;
+
+  LaneSplit(Program& prog, const Options& o, NameGen& g) : p(prog), opts(o), gen(g), isz(o.int_size()) {}
+
+  // the sum loop: a sequential loop over [0, K) whose body is `t = t + e`, all d-dependent accesses unit-stride
+  bool sum_loop(const S& s, int* vec) {
+    if (!(s->k == Stmt::For && s->map.k == GpuMap::None && !s->unroll && s->step == 1 && s->lo->k == Expr::Int && s->lo->iv == 0 &&
+          s->hi->k == Expr::Int && s->body.size() == 1))
+      return false;
+    const S& a = s->body[0];
+    if (!(a->k == Stmt::Assign && a->dst->k == Expr::Var && a->dst->ty.is_scalar() && is_float(a->dst->ty.sz))) return false;
+    if (!(a->expr->k == Expr::BinOpE && a->expr->bop == BinOp::Add)) return false;
+    const E &l = a->expr->args[0], &r = a->expr->args[1];
+    E term;
+    if (l->k == Expr::Var && l->name == a->dst->name) term = r;
+    else if (r->k == Expr::Var && r->name == a->dst->name) term = l;
+    if (!term || mentions(term, a->dst->name)) return false;
+    int v = 0, loads = 0;
+    bool ok = true;
+    visit_exprs(term, [&](const E& x) {
+      if (x->k == Expr::Call || x->k == Expr::AddrOf) ok = false;
+      if (x->k != Expr::Index) return;
+      if (!mentions(x->args[1], s->id)) return;
+      E rest;
+      if (!affine_unit(x->args[1], s->id, &rest)) { ok = false; return; }
+      int w = elem_bytes(x->ty.sz) == 4 ? 4 : elem_bytes(x->ty.sz) == 8 ? 2 : 0;
+      if (w == 0) { ok = false; return; }
+      v = v == 0 ? w : std::min(v, w);
+      ++loads;
+    });
+    if (!ok || loads < 2 || s->hi->iv % (v * G) != 0 || s->hi->iv < 4 * v * G) return false;
+    *vec = v;
+    return true;
+  }
+
+  bool apply(Kernel& k, const StmtP& launch) {
+    if (k.body.size() != 1) return false;
+    const S& root = k.body[0];
+    if (!(root->k == Stmt::For && root->map.k == GpuMap::ThreadBlock && root->map.dim == 0 && root->step == 1 &&
+          root->lo->k == Expr::Int && root->lo->iv == 0 && root->hi->k == Expr::Int))
+      return false;
+    int64_t N = root->hi->iv;
+    if (N < 4096 || k.grid.y != 1 || k.grid.z != 1 || k.block.y != 1 || k.block.z != 1) return false;  // small launches gain nothing
+    int pos = -1, vec = 0;
+    for (size_t q = 0; q < root->body.size(); ++q) {
+      const S& st = root->body[q];
+      int v = 0;
+      if (sum_loop(st, &v)) {
+        if (pos >= 0) return false;
+        pos = (int)q;
+        vec = v;
+        continue;
+      }
+      bool simple = st->k == Stmt::Def || (st->k == Stmt::Assign && (st->dst->k == Expr::Index || st->dst->k == Expr::Var));
+      if (!simple) return false;
+      if (pos < 0 && st->k == Stmt::Assign && st->dst->k == Expr::Index) return false;  // stores before the sum: keep it simple
+    }
+    if (pos < 0) return false;
+    const S& loop = root->body[pos];
+    Type ity = Type::scalar(isz);
+    Name gi = gen.fresh(root->id.s + "_lane"), g = gen.fresh("g"), d0 = gen.fresh(loop->id.s + "_c"), u = gen.fresh(loop->id.s + "_u");
+    E giv = mk_var(gi, ity), gv = mk_var(g, ity);
+    Stmts body;
+    body.push_back(mk_def(root->id, ity, mk_binop(BinOp::FloorDiv, giv, mk_int(G, isz), ity), root->i));
+    body.push_back(mk_def(g, ity, mk_binop(BinOp::Rem, giv, mk_int(G, isz), ity), root->i));
+    for (int q = 0; q < pos; ++q) body.push_back(root->body[q]);
+    // d = (d0 * G + g) * V + u
+    E d = mk_binop(BinOp::Add,
+                   mk_binop(BinOp::Mul, mk_binop(BinOp::Add, mk_binop(BinOp::Mul, mk_var(d0, ity), mk_int(G, isz), ity), gv, ity),
+                            mk_int(vec, isz), ity),
+                   mk_var(u, ity), ity);
+    Stmts ib;
+    ib.push_back(mk_def(loop->id, ity, d, loop->i));
+    ib.push_back(loop->body[0]);
+    auto inner = std::const_pointer_cast<Stmt>(std::static_pointer_cast<const Stmt>(
+        mk_for(u, mk_int(0, isz), mk_int(vec, isz), 1, ib, LoopPar(), loop->i)));
+    inner->unroll = true;
+    auto outer = clone(loop);
+    outer->id = d0;
+    outer->hi = mk_int(loop->hi->iv / (vec * G), isz);
+    outer->body = {S(inner)};
+    body.push_back(outer);
+    const E& t = loop->body[0]->dst;
+    body.push_back(mk_assign(t, mk_raw("parpy_sum8(" + t->name.str() + ")", t->ty)));
+    Stmts stores;
+    for (size_t q = pos + 1; q < root->body.size(); ++q) {
+      const S& st = root->body[q];
+      if (st->k == Stmt::Assign && st->dst->k == Expr::Index) stores.push_back(st);
+      else {
+        if (!stores.empty()) return false;  // a definition after a store: not the shape this pass handles
+        body.push_back(st);
+      }
+    }
+    if (!stores.empty()) body.push_back(mk_if(mk_binop(BinOp::Eq, gv, mk_int(0, isz), Type::scalar(ElemSize::Bool)), stores, {}));
+    auto nr = clone(root);
+    nr->id = gi;
+    nr->hi = mk_int(N * G, isz);
+    nr->body = body;
+    int64_t tpb = root->map.tpb;
+    nr->map.n = (N * G + WAVE_SIZE - 1) / WAVE_SIZE * WAVE_SIZE;
+    k.body = {S(nr)};
+    k.grid.x = (nr->map.n + tpb - 1) / tpb;
+    launch->grid = k.grid;
+    return true;
+  }
+
+  void run() {
+    Stmts host;
+    for (auto& s : p.host) {
+      if (s->k != Stmt::Launch) { host.push_back(s); continue; }
+      Kernel* k = nullptr;
+      for (auto& kk : p.kernels)
+        if (kk.name == s->fname) k = &kk;
+      auto ns = std::make_shared<Stmt>(*s);
+      if (k && !k->opaque_body) apply(*k, ns);
+      host.push_back(ns);
+    }
+    p.host = host;
+  }
+};
+
 }  // namespace
 
 void hip_optimize(Program& p, const Options& opts, NameGen& gen) {
   if (opts.opt_gather_transpose) GatherTranspose(p, opts, gen).run();
+  if (opts.opt_lane_split && !opts.opt_mfma_sddmm) LaneSplit(p, opts, gen).run();
   for (auto& k : p.kernels) {
     if (k.opaque_body) { k.aligned_params = opts.assume_aligned; continue; }
     Pass pass(k, opts, gen);

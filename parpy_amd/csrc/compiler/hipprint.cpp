@@ -146,6 +146,13 @@ __device__ __forceinline__ T parpy_block_reduce(T v, T neutral, T* slots, bool s
   }
   return v;
 }
+// sum over each aligned group of 8 lanes; every lane of the group receives it
+template <class T> __device__ __forceinline__ T parpy_sum8(T v) {
+  v = v + parpy_dpp<0xB1>(v);   // lane ^ 1
+  v = v + parpy_dpp<0x4E>(v);   // lane ^ 2
+  v = v + parpy_dpp<0x141>(v);  // the other quad of the 8-lane half row
+  return v;
+}
 typedef float parpy_f32x4 __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ int parpy_lane_id() { return (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)); }
 // dst[c][r] = src[r][c] for a ROWS x COLS matrix in 64 x 64 tiles: a 256-thread workgroup reads

@@ -206,6 +206,15 @@ def test_sddmm_kernels_compile():
     C2 = {"rows": oracle.csr_rows(crows2), "cols": cols2, "values": vals2, "nnz": len(cols2)}
     st = compiles(parpy.print_compiled(W.sddmm_coo, [A2, B2, C2, np.zeros_like(vals2), 1.5, 2.0], opts_for({"nnz": parpy.threads(len(cols2))})))
     assert "parpy_transpose_tile<float, 64, 256>(" in st and launch(st)[0] == ("4", "1", "1", "256", "1", "1")
+    # at full size eight lanes share one non-zero: the launch grows eightfold and lane 0 of a group stores
+    A3, B3, crows3, cols3, vals3 = W.make_sddmm(1024, 128, 0.01)
+    C3 = {"rows": oracle.csr_rows(crows3), "cols": cols3, "values": vals3, "nnz": len(cols3)}
+    n3 = len(cols3)
+    sl = compiles(parpy.print_compiled(W.sddmm_coo, [A3, B3, C3, np.zeros_like(vals3), 1.5, 2.0], opts_for({"nnz": parpy.threads(n3).tpb(256)})))
+    assert "parpy_sum8(t_" in sl and launch(sl)[1][0] == str((n3 * 8 + 255) // 256)
+    sn = compiles(parpy.print_compiled(W.sddmm_coo, [A3, B3, C3, np.zeros_like(vals3), 1.5, 2.0],
+                                       opts_for({"nnz": parpy.threads(n3).tpb(256)}, opt_lane_split=False)))
+    assert "parpy_sum8(t_" not in sn and launch(sn)[1][0] == str((n3 + 255) // 256)
     s = compiles(parpy.print_compiled(W.sddmm_decompress_csr, [crows, np.zeros_like(cols), 128],
                                       opts_for({"N": parpy.threads(128), "M": parpy.threads(64)})))
     assert launch(s) == [("1", "128", "1", "64", "1", "1")]

@@ -215,7 +215,8 @@ def test_forward_all_states_unreachable_gives_neg_inf():
 
 
 # ---------------------------------------------------------------- SDDMM
-@pytest.mark.parametrize("flags", [{}, {"opt_mfma_sddmm": True}, {"opt_gather_transpose": False}], ids=["default", "mfma", "no-transpose"])
+@pytest.mark.parametrize("flags", [{}, {"opt_mfma_sddmm": True}, {"opt_gather_transpose": False}, {"opt_lane_split": False}],
+                         ids=["default", "mfma", "no-transpose", "no-lane-split"])
 @pytest.mark.parametrize("n,k,density", [(256, 32, 0.05), (8192, 128, 0.01)])
 def test_sddmm(n, k, density, flags):
     A, B, crows, cols, vals = W.make_sddmm(n, k, density)
