@@ -90,8 +90,8 @@ def _raise_last_error(lib, filepath):
     if l0 > 0 and filepath:
         lines = [linecache.getline(filepath, n).rstrip("\n") for n in range(l0, max(l0, l1) + 1)]
         excerpt = "\n".join(f"{n:4d} | {t}" for n, t in zip(range(l0, l1 + 1), lines) if t)
-        where = f"on line {l0}" if l0 == l1 else f"on lines {l0}-{l1}"
-        msg = f"{msg}\nIn file {filepath} {where}:\n{excerpt}"
+        where = f"line {l0}" if l0 == l1 else f"lines {l0}-{l1}"
+        msg = f"{msg}\n\nOn {where} of file {filepath}:\n{excerpt}"
     exc = {0: RuntimeError, 1: TypeError, 2: NameError}.get(kind, RuntimeError)
     raise exc(msg)
 

@@ -988,7 +988,7 @@ FunDef specialize(const ParsedFun& pf, const std::vector<ArgDesc>& args, const O
   if (args.size() != f.params.size())
     fail_ty(f.i, "Function " + f.id.s + " expected " + std::to_string(f.params.size()) + " arguments, but received " +
                      std::to_string(args.size()) + ".");
-  if (has_return(f.body)) fail_rt(f.i, "The main function " + f.id.s + " cannot contain a return statement.");
+  if (has_return(f.body)) fail_rt(f.i, "The called function " + f.id.s + " cannot return a value");  // src/py/no_return.rs:10-16
 
   Specializer sp(opts, gen);
   for (size_t k = 0; k < args.size(); ++k)

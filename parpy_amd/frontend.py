@@ -87,8 +87,15 @@ class _Converter:
         return f"@{l0}:{c0}:{l1}:{c1}"
 
     def err(self, node, msg):
+        """Report `msg` with the source lines of `node`, the way the reference does
+        (src/utils/info.rs:90-121): 'On line(s) a-b of file f:' followed by the lines."""
+        import linecache
         l0 = getattr(node, "lineno", 0) + self.line_ofs
-        raise FrontendError(f"{msg} (file {self.filepath}, line {l0})")
+        l1 = (getattr(node, "end_lineno", None) or getattr(node, "lineno", 0)) + self.line_ofs
+        where = f"line {l0}" if l0 == l1 else f"lines {l0}-{l1}"
+        lines = [linecache.getline(self.filepath, n).rstrip("\n") for n in range(l0, l1 + 1)]
+        excerpt = "\n".join(f"{n:4d} | {t}" for n, t in zip(range(l0, l1 + 1), lines) if t)
+        raise FrontendError(f"{msg}\n\nOn {where} of file {self.filepath}:\n{excerpt}")
 
     def eval_name(self, src):
         return eval(src, self.globs, self.locs)

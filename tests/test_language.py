@@ -350,3 +350,71 @@ def test_slice_statements_on_device(spec):
     spec[0](*want)
     parpy.jit(spec[0])(*got, opts=opts_for(SLICE_PAR))
     assert np.allclose(got[-1], want[-1], atol=1e-4)
+
+
+# ---------------------------------------------------------------- constructs rejected when the function is parsed
+def test_unsupported_statements_report_their_lines():
+    """test/test_unsupported.py of the reference: the message names the lines of the offending statement."""
+    import inspect
+    here = inspect.currentframe().f_lineno
+    with pytest.raises(RuntimeError, match=rf"lines {here + 5}-{here + 9}"):
+        @parpy.jit
+        def while_else(x, y, N):
+            i = 0
+            while i < N:
+                y[i] = x[i]
+                i += 1
+            else:
+                y[i] = 0.0
+    here = inspect.currentframe().f_lineno
+    with pytest.raises(RuntimeError, match=rf"lines {here + 4}-{here + 7}"):
+        @parpy.jit
+        def for_else(x, y, N):
+            for i in range(N):
+                y[i] = x[i]
+            else:
+                y[0] += 1
+    here = inspect.currentframe().f_lineno
+    with pytest.raises(RuntimeError, match=rf"lines {here + 4}-{here + 5}"):
+        @parpy.jit
+        def with_context():
+            with 5:
+                pass
+    here = inspect.currentframe().f_lineno
+    with pytest.raises(RuntimeError, match=rf"lines {here + 4}-{here + 5}"):
+        @parpy.jit
+        def with_as():
+            with parpy.gpu as x:
+                a = x + 1
+    with pytest.raises(RuntimeError, match=r"Empty return statements are not supported"):
+        @parpy.jit
+        def empty_return():
+            return
+
+
+def test_entry_function_rules():
+    @parpy.jit
+    def dict_arg(a):
+        with parpy.gpu:
+            a["x"] = a["y"]
+    # (without a GPU the call stops at backend resolution, as in the reference's own test)
+    with pytest.raises(RuntimeError, match=r"(.*non-string key.*)|(.*backend.*not available.*)"):
+        dict_arg({'x': 2, 'y': 4, 3: 5}, opts=opts_for({}))
+    o = parpy.CompileOptions()
+    with pytest.raises(RuntimeError, match=r".*number of thread blocks per cluster must be a power of two.*"):
+        o.max_thread_blocks_per_cluster = 3
+
+    @parpy.jit
+    def f_return(x):
+        with parpy.gpu:
+            y = sum(x[:])
+            return y
+    with pytest.raises(RuntimeError, match=r"The called function f_return cannot return a value"):
+        parpy.print_compiled(f_return, [np.ndarray(10)], opts_for({}))
+
+    @parpy.jit
+    def fun_with_args(x, y):
+        with parpy.gpu:
+            x[:] += y[:]
+    with pytest.raises(RuntimeError, match="Missing required keyword argument opts in call to fun_with_args"):
+        fun_with_args(np.ndarray((10,), dtype=np.float32), np.ndarray((10,), dtype=np.float32))
