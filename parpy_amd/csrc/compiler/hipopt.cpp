@@ -1353,19 +1353,26 @@ struct LaneSplit {
 
   LaneSplit(Program& prog, const Options& o, NameGen& g) : p(prog), opts(o), gen(g), isz(o.int_size()) {}
 
-  // the sum loop: a sequential loop over [0, K) whose body is `t = t + e`, all d-dependent accesses unit-stride
-  bool sum_loop(const S& s, int* vec) {
+  // the sum loop: a sequential loop over [0, K) whose body is `acc = acc + e`, where acc is a scalar
+  // variable or an array element that does not depend on d, and all d-dependent accesses are unit-stride
+  bool sum_loop(const S& s, int* vec, E* term_out) {
     if (!(s->k == Stmt::For && s->map.k == GpuMap::None && !s->unroll && s->step == 1 && s->lo->k == Expr::Int && s->lo->iv == 0 &&
           s->hi->k == Expr::Int && s->body.size() == 1))
       return false;
     const S& a = s->body[0];
-    if (!(a->k == Stmt::Assign && a->dst->k == Expr::Var && a->dst->ty.is_scalar() && is_float(a->dst->ty.sz))) return false;
+    if (a->k != Stmt::Assign) return false;
+    const E& acc = a->dst;
+    bool scalar_acc = acc->k == Expr::Var && acc->ty.is_scalar();
+    bool elem_acc = acc->k == Expr::Index && acc->args[0]->k == Expr::Var && !mentions(acc->args[1], s->id) && !has_load(acc->args[1]);
+    if (!(scalar_acc || elem_acc) || !is_float(acc->ty.sz)) return false;
     if (!(a->expr->k == Expr::BinOpE && a->expr->bop == BinOp::Add)) return false;
     const E &l = a->expr->args[0], &r = a->expr->args[1];
     E term;
-    if (l->k == Expr::Var && l->name == a->dst->name) term = r;
-    else if (r->k == Expr::Var && r->name == a->dst->name) term = l;
-    if (!term || mentions(term, a->dst->name)) return false;
+    if (expr_eq(l, acc)) term = r;
+    else if (expr_eq(r, acc)) term = l;
+    if (!term) return false;
+    const Name& acc_name = scalar_acc ? acc->name : acc->args[0]->name;
+    if (mentions(term, acc_name)) return false;
     int v = 0, loads = 0;
     bool ok = true;
     visit_exprs(term, [&](const E& x) {
@@ -1379,8 +1386,9 @@ struct LaneSplit {
       v = v == 0 ? w : std::min(v, w);
       ++loads;
     });
-    if (!ok || loads < 2 || s->hi->iv % (v * G) != 0 || s->hi->iv < 4 * v * G) return false;
+    if (!ok || loads < 1 || s->hi->iv % (v * G) != 0 || s->hi->iv < 4 * v * G) return false;
     *vec = v;
+    *term_out = term;
     return true;
   }
 
@@ -1393,28 +1401,58 @@ struct LaneSplit {
     int64_t N = root->hi->iv;
     if (N < 4096 || k.grid.y != 1 || k.grid.z != 1 || k.block.y != 1 || k.block.z != 1) return false;  // small launches gain nothing
     int pos = -1, vec = 0;
+    E term;
     for (size_t q = 0; q < root->body.size(); ++q) {
       const S& st = root->body[q];
       int v = 0;
-      if (sum_loop(st, &v)) {
+      E t;
+      if (sum_loop(st, &v, &t)) {
         if (pos >= 0) return false;
         pos = (int)q;
         vec = v;
+        term = t;
         continue;
       }
       bool simple = st->k == Stmt::Def || (st->k == Stmt::Assign && (st->dst->k == Expr::Index || st->dst->k == Expr::Var));
       if (!simple) return false;
-      if (pos < 0 && st->k == Stmt::Assign && st->dst->k == Expr::Index) return false;  // stores before the sum: keep it simple
     }
     if (pos < 0) return false;
     const S& loop = root->body[pos];
+    const E& acc = loop->body[0]->dst;
+    bool elem_acc = acc->k == Expr::Index;
+    // an array element as accumulator: nothing else in the iteration may touch that array but plain
+    // stores to the very element in front of the loop (its initialisation)
+    if (elem_acc)
+      for (size_t q = 0; q < root->body.size(); ++q) {
+        if ((int)q == pos) continue;
+        const S& st = root->body[q];
+        bool init = (int)q < pos && st->k == Stmt::Assign && expr_eq(st->dst, acc) && !mentions(st->expr, acc->args[0]->name);
+        if (init) continue;
+        bool touches = false;
+        auto scan = [&](const E& e) { if (e && mentions(e, acc->args[0]->name)) touches = true; };
+        scan(st->dst); scan(st->expr);
+        if (touches) return false;
+      }
+    for (int q = 0; q < pos; ++q)   // other stores in front of the sum would be repeated by every lane of a group: harmless, same value
+      if (root->body[q]->k == Stmt::Assign && root->body[q]->dst->k == Expr::Index && !expr_eq(root->body[q]->dst, acc)) return false;
     Type ity = Type::scalar(isz);
     Name gi = gen.fresh(root->id.s + "_lane"), g = gen.fresh("g"), d0 = gen.fresh(loop->id.s + "_c"), u = gen.fresh(loop->id.s + "_u");
     E giv = mk_var(gi, ity), gv = mk_var(g, ity);
+    E lane0 = mk_binop(BinOp::Eq, gv, mk_int(0, isz), Type::scalar(ElemSize::Bool));
     Stmts body;
     body.push_back(mk_def(root->id, ity, mk_binop(BinOp::FloorDiv, giv, mk_int(G, isz), ity), root->i));
     body.push_back(mk_def(g, ity, mk_binop(BinOp::Rem, giv, mk_int(G, isz), ity), root->i));
-    for (int q = 0; q < pos; ++q) body.push_back(root->body[q]);
+    for (int q = 0; q < pos; ++q) {
+      const S& st = root->body[q];
+      if (st->k == Stmt::Assign && st->dst->k == Expr::Index) body.push_back(mk_if(lane0, {st}, {}));
+      else body.push_back(st);
+    }
+    E t = acc;
+    if (elem_acc) {
+      Name tn = gen.fresh("part");
+      body.push_back(mk_def(tn, acc->ty, mk_float(0.0, acc->ty.sz), loop->i));
+      t = mk_var(tn, acc->ty);
+    }
     // d = (d0 * G + g) * V + u
     E d = mk_binop(BinOp::Add,
                    mk_binop(BinOp::Mul, mk_binop(BinOp::Add, mk_binop(BinOp::Mul, mk_var(d0, ity), mk_int(G, isz), ity), gv, ity),
@@ -1422,7 +1460,7 @@ struct LaneSplit {
                    mk_var(u, ity), ity);
     Stmts ib;
     ib.push_back(mk_def(loop->id, ity, d, loop->i));
-    ib.push_back(loop->body[0]);
+    ib.push_back(mk_assign(t, mk_binop(BinOp::Add, t, term, t->ty), loop->i));
     auto inner = std::const_pointer_cast<Stmt>(std::static_pointer_cast<const Stmt>(
         mk_for(u, mk_int(0, isz), mk_int(vec, isz), 1, ib, LoopPar(), loop->i)));
     inner->unroll = true;
@@ -1431,9 +1469,13 @@ struct LaneSplit {
     outer->hi = mk_int(loop->hi->iv / (vec * G), isz);
     outer->body = {S(inner)};
     body.push_back(outer);
-    const E& t = loop->body[0]->dst;
     body.push_back(mk_assign(t, mk_raw("parpy_sum8(" + t->name.str() + ")", t->ty)));
     Stmts stores;
+    if (elem_acc) {
+      // a group that lies wholly in one lane-0 store: the synchronisation between the initialising store
+      // and this read-modify-write is program order of lane 0
+      stores.push_back(mk_assign(acc, mk_binop(BinOp::Add, acc, t, acc->ty), loop->i));
+    }
     for (size_t q = pos + 1; q < root->body.size(); ++q) {
       const S& st = root->body[q];
       if (st->k == Stmt::Assign && st->dst->k == Expr::Index) stores.push_back(st);
@@ -1442,7 +1484,7 @@ struct LaneSplit {
         body.push_back(st);
       }
     }
-    if (!stores.empty()) body.push_back(mk_if(mk_binop(BinOp::Eq, gv, mk_int(0, isz), Type::scalar(ElemSize::Bool)), stores, {}));
+    if (!stores.empty()) body.push_back(mk_if(lane0, stores, {}));
     auto nr = clone(root);
     nr->id = gi;
     nr->hi = mk_int(N * G, isz);

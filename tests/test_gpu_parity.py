@@ -70,6 +70,15 @@ def test_reductions(fn, case):
     assert np.allclose(out, want, atol=tol, rtol=1e-5), (np.abs(out - want).max(), fn.__name__, case[0])
 
 
+@pytest.mark.parametrize("lane_split", [True, False])
+def test_one_thread_per_row_on_many_rows(lane_split):
+    """4096 rows summed by one thread each: eight lanes share a row when the lane-group pass is on."""
+    x = np.random.default_rng(9).uniform(-1, 1, (4096, 512)).astype(np.float32)
+    out = np.zeros(4096, dtype=np.float32)
+    parpy.jit(K.sum_rows)(x, out, 4096, opts=opts_for({'outer': parpy.threads(4096)}, opt_lane_split=lane_split))
+    assert np.allclose(out, x.astype(np.float64).sum(axis=1), atol=1e-4, rtol=1e-5)
+
+
 @pytest.mark.parametrize("threads", [64, 2048])
 def test_strided_reduction(threads):
     N, M = 10, 4096
