@@ -1,6 +1,6 @@
 """Benchmark of the compiled hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload hmm7|hmm5|rowsum|softmax|sddmm]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload hmm7|hmm5|hmm5ref|rowsum|softmax|sddmm|copy]
 
 A step is one pass of the compiled function over one batch of seeded synthetic
 input that is already resident in HBM.  The default workload is the headline
@@ -77,6 +77,44 @@ def bench_hmm(k, args, torch, parpy, W):
                      "frac": alg_bytes / (kernel_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None,
                      "kernel_ms": kernel_ms, "algorithmic_bytes": alg_bytes},
         "cpu_baseline": cpu,
+    }
+
+
+def bench_hmm_ref(args, torch, parpy, W):
+    """The reference's own 5-mer model (16 duration layers x 1024 k-mers = 16384 states) on its 100
+    recorded reads, tables from tests/golden: the configuration its benchmark validates
+    (benchmarks/forward.py:481-518).  Results are checked against the expected log-likelihoods."""
+    import numpy as np
+    g = os.path.join(ROOT, "tests", "golden")
+    hmm, seqs = W.load_reference_model(os.path.join(g, "hmm_5mer_model.npz"), os.path.join(g, "hmm_signals.npz"))
+    want = np.loadtxt(os.path.join(g, "hmm_5mer_expected.txt"), dtype=np.float32)
+    S, n = hmm["num_states"], seqs["num_instances"]
+    hd, sd = W.to_device(hmm), W.to_device(seqs)
+    a1 = torch.zeros((n, S), dtype=torch.float32, device="cuda")
+    a2 = torch.zeros_like(a1)
+    res = torch.zeros(n, dtype=torch.float32, device="cuda")
+    nthreads = min(S, args.state_threads)
+    opts = parpy.par({"inst": parpy.threads(n), "state": parpy.threads(nthreads)})
+    _apply_opt_flags(opts, args)
+    fn = lambda: W.forward_kernel(hd, sd, a1, a2, res, opts=opts)
+    timed = lambda: parpy.time_call(W.forward_kernel, hd, sd, a1, a2, res, opts=opts)
+    wall, dev = _events_ms(fn, timed, args.steps, args.warmup, torch)
+    got = res.cpu().numpy()
+    assert np.allclose(got, want, atol=1e-5, rtol=1e-5), float(np.abs(got - want).max())
+    steps_total = int((seqs["lens"] - 1).sum())
+    # per (read, step): alpha read + alpha write (4S each), one emission row of S/16 k-mers, the observation byte
+    alg_bytes = (8 * S + 4 * (S // 16) + 1) * steps_total
+    kernel_ms = float(np.median(dev))
+    return {
+        "metric": "HMM-forward reference 5-mer model ms/batch + achieved HBM GB/s (% of peak), 1xMI355X",
+        "value": wall, "unit": "ms/batch", "ms_per_step": wall, "higher_is_better": False, "dtype": "f32",
+        "config": {"workload": "hmm_forward_reference_5mer_model", "states": S, "reads": n, "min_len": int(seqs["lens"].min()),
+                   "max_len": int(seqs["lens"].max()), "total_steps": steps_total, "state_threads": nthreads,
+                   "mean_loglik": float(got.mean())},
+        "roofline": {"bound": "hbm", "achieved": alg_bytes / (kernel_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": alg_bytes / (kernel_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None,
+                     "kernel_ms": kernel_ms, "algorithmic_bytes": alg_bytes},
+        "cpu_baseline": None,
     }
 
 
@@ -220,7 +258,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="hmm7", choices=["hmm7", "hmm5", "rowsum", "softmax", "sddmm", "copy"])
+    ap.add_argument("--workload", default="hmm7", choices=["hmm7", "hmm5", "hmm5ref", "rowsum", "softmax", "sddmm", "copy"])
     ap.add_argument("--state-threads", type=int, default=1024)
     ap.add_argument("--use-graphs", type=int, default=0, help="replay the launches of a run from a HIP graph (host-hoisted time loops)")
     ap.add_argument("--inner-threads", type=int, default=None)
@@ -247,6 +285,8 @@ def main():
         r = bench_hmm(7, args, torch, parpy, W)
     elif args.workload == "hmm5":
         r = bench_hmm(5, args, torch, parpy, W)
+    elif args.workload == "hmm5ref":
+        r = bench_hmm_ref(args, torch, parpy, W)
     elif args.workload == "rowsum":
         r = bench_rowsum(args, torch, parpy, W)
     elif args.workload == "softmax":
@@ -260,7 +300,7 @@ def main():
     if default_cfg and not args.reg_budget:
         r["roofline"]["traffic"] = _profiled_traffic(args.workload)
     r.update({"n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "scaling": "weak", "vs_baseline": None,
-              "data": "synthetic"})
+              "data": "reference fixtures (tests/golden)" if args.workload == "hmm5ref" else "synthetic"})
     print(json.dumps(r))
 
 

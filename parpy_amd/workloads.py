@@ -289,6 +289,53 @@ def synthetic_hmm(k, n_inst=100, min_len=5000, max_len=15000, seed=SEED, emissio
     return hmm, seqs
 
 
+def load_reference_model(model_npz, signals_npz):
+    """Kernel inputs for `forward_kernel` from the reference's model and signal tables (as re-packed
+    from its HDF5 files): the layout work of test/test_forward.py:31-77 and
+    benchmarks/forward.py:232-312.
+
+    model: `k`, `obs` [101, 4^k] emission probabilities indexed by the k-mer read in reverse base
+    order, `trans` 4 x 4^k successor probabilities, `duration` [16], `tail_factor`.
+    Returned tables are natural logarithms in float32: `trans1` [4^k, 4], `trans2` [16],
+    `output_prob` [101, 4^k] re-indexed to forward base order, `initial_prob` uniform over the
+    first duration layer and -inf elsewhere, `gamma` = log tail, `synthetic_248` = log(1 - tail).
+    Signals are concatenated int levels with per-read lengths; they become a zero-padded int8 matrix.
+    """
+    m = np.load(model_npz)
+    k = int(m["k"])
+    nk = 4 ** k
+    # index of each k-mer with its base-4 digits reversed
+    idx = np.arange(nk)
+    rev = np.zeros(nk, dtype=np.int64)
+    for _ in range(k):
+        rev = rev * 4 + idx % 4
+        idx = idx // 4
+    with np.errstate(divide="ignore"):
+        # logarithms in the precision the tables are stored in, as the reference takes them
+        log_obs = np.log(m["obs"])
+        log_trans = np.log(m["trans"])
+    tail = float(m["tail_factor"])
+    init = np.full(16 * nk, -np.inf, dtype=np.float32)
+    init[:nk] = np.float32(-np.log(float(nk)))
+    hmm = {
+        "trans1": np.ascontiguousarray(log_trans.reshape(4, nk).T, dtype=np.float32),
+        "trans2": np.log(m["duration"]).astype(np.float32),
+        "output_prob": np.ascontiguousarray(log_obs[:, rev], dtype=np.float32),
+        "initial_prob": init,
+        "gamma": np.float32(np.log(tail)),
+        "synthetic_248": np.float32(np.log1p(-tail)),
+        "num_states": 16 * nk,
+    }
+    s = np.load(signals_npz)
+    lens = np.asarray(s["lens"], dtype=np.int64)
+    ends = np.cumsum(lens)
+    data = np.zeros((len(lens), int(lens.max())), dtype=np.int8)
+    for i, (e, n) in enumerate(zip(ends, lens)):
+        data[i, :n] = s["samples"][e - n:e]
+    seqs = {"data": data, "lens": lens, "maxlen": int(lens.max()), "num_instances": len(lens)}
+    return hmm, seqs
+
+
 def to_device(d, device="cuda"):
     """Move the arrays of a workload dict to torch tensors on `device`; ints stay Python ints."""
     import torch

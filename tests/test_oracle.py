@@ -156,3 +156,16 @@ def test_sddmm_against_dense_product():
     eye = np.eye(8, dtype=np.float32)
     assert np.allclose(oracle.sddmm(eye, eye, np.arange(8), np.arange(8)), 1.0)
     assert np.allclose(oracle.sddmm(eye, eye, np.arange(8), (np.arange(8) + 1) % 8), 0.0)
+
+
+def test_product_side_model_loader_agrees_with_the_oracle(golden_dir):
+    """Two independent restatements of the reference's table layout (test/test_forward.py:31-77)."""
+    import os
+    from parpy_amd import workloads as W
+    for k in (3, 5):
+        paths = (os.path.join(golden_dir, f"hmm_{k}mer_model.npz"), os.path.join(golden_dir, "hmm_signals.npz"))
+        a, b = oracle.reference_model_tables(*paths), W.load_reference_model(*paths)
+        for da, db in zip(a, b):
+            assert sorted(da) == sorted(db)
+            for key in da:
+                assert np.array_equal(np.asarray(da[key]), np.asarray(db[key])), (k, key)
