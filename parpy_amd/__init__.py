@@ -127,6 +127,8 @@ def clear_cache():
     """Clear the cached code objects and the in-memory function cache."""
     from .compile import clear_cache as _clear
     global _fun_cache
+    for f in _ir_asts:
+        getattr(f, "_seen_calls", {}).clear()
     _clear()
     _fun_cache = {}
 
@@ -214,6 +216,45 @@ def external(ext_name, backend, target, header=None, parallelize=LoopPar()):
     return external_wrap
 
 
+def _call_signature(args):
+    """(signature, device pointers, all 16-byte aligned) of a call whose arrays are all contiguous
+    torch tensors on the device and whose other arguments are plain scalars; None for anything else.
+    Two calls with equal signatures specialise to the same code and differ only in the pointers."""
+    import sys
+    torch = sys.modules.get("torch")
+    if torch is None:
+        return None
+    sig, ptrs, aligned = [], [], True
+    for a in args:
+        if type(a) is dict:
+            try:
+                items = sorted(a.items())
+            except TypeError:      # keys of mixed types: let the validation report it
+                return None
+        else:
+            items = ((None, a),)
+        for k, v in items:
+            t = type(v)
+            if t is torch.Tensor:
+                if v.dim() == 0:
+                    if v.is_cuda:
+                        return None
+                    sig.append((k, v.dtype, v.item()))
+                elif v.is_cuda and v.is_contiguous() and not v.requires_grad:
+                    p = v.data_ptr()
+                    ptrs.append(p)
+                    aligned = aligned and p % 16 == 0
+                    sig.append((k, v.dtype, v.shape))
+                else:
+                    return None
+            elif t is int or t is float or t is bool:
+                sig.append((k, t, v))
+            else:
+                return None
+        sig.append(len(items))
+    return tuple(sig), ptrs, aligned
+
+
 def jit(fun):
     """Prepare `fun` for JIT compilation: parse once now, specialise on the arguments of each call."""
     from .validate import check_arguments
@@ -223,10 +264,30 @@ def jit(fun):
     locs = inspect.currentframe().f_back.f_locals
     ir_ast = _convert_python_function_to_ir(fun, (globs, locs))
 
+    # calls seen before: (argument signature, alignment, options state) -> compiled wrapper; a hit
+    # skips validation, buffer wrapping and key printing and goes straight to the launch plan
+    seen = {}
+
     @functools.wraps(fun)
     def inner(*args, **kwargs):
+        opts = kwargs.get("opts")
+        if len(kwargs) == 1 and type(opts) is CompileOptions:
+            call = _call_signature(args)
+            if call is not None:
+                key = (call[0], call[2], opts._fast_key())
+                hit = seen.get(key)
+                if hit is not None:
+                    return hit.run_pointers(call[1])
+        else:
+            call = None
         opts = backend._resolve_backend(_check_kwargs(kwargs, fun.__name__), True)
-        args = check_arguments(args, opts, True)
-        _compile_function(ir_ast, args, opts)(*args)
+        checked = check_arguments(args, opts, True)
+        wrap_fn = _compile_function(ir_ast, checked, opts)
+        wrap_fn(*checked)
+        if call is not None and getattr(wrap_fn, "run_pointers", None) is not None:
+            if len(seen) > 256:
+                seen.clear()
+            seen[(call[0], call[2], opts._fast_key())] = wrap_fn   # (backend resolution may have touched opts)
     _ir_asts[inner] = ir_ast
+    inner._seen_calls = seen
     return inner

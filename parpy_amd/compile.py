@@ -134,7 +134,14 @@ def get_wrapper(name, key, plan_text, opts):
             raise RuntimeError(f"{lib.parpy_get_error_message().decode('ascii', 'replace')}")
         return ms.value
 
+    def run_pointers(ptrs):
+        """Run on device pointers that were validated before (same order as `wrapper` derives them)."""
+        arr = (ctypes.c_void_p * max(1, len(ptrs)))(*ptrs)
+        if lib.parpy_hip_plan_run(plan, arr, len(ptrs)) != 0:
+            raise RuntimeError(f"{lib.parpy_get_error_message().decode('ascii', 'replace')}")
+
     wrapper.__name__ = name
+    wrapper.run_pointers = run_pointers
     wrapper.timed = timed
     wrapper.plan = plan
     wrapper.launch_count = lambda: lib.parpy_hip_plan_launch_count(plan)

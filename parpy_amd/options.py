@@ -200,8 +200,21 @@ class LoopPar:
     __str__ = __repr__
 
 
+_options_clock = [0]
+
+
 class CompileOptions:
     """src/option.rs:14-108; __str__ feeds the in-memory cache key (python/parpy/key.py:29-30)."""
+
+    def __setattr__(self, name, value):
+        # every assignment to any options object gets a stamp that no other assignment has:
+        # (stamp, parallelize) identifies the state of an options object cheaply
+        _options_clock[0] += 1
+        object.__setattr__(self, "_stamp", _options_clock[0])
+        object.__setattr__(self, name, value)
+
+    def _fast_key(self):
+        return (self._stamp, tuple((k, p.nthreads, p.reduction, p._tpb) for k, p in self.parallelize.items()))
 
     def __init__(self):
         self.parallelize = {}

@@ -390,3 +390,34 @@ def test_aliases_that_may_coincide(noalias):
     ad, bd = torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda()
     parpy.jit(K.alias_maybe_same)(ad, bd, 4, 64, 3, opts=opts_for({'N': parpy.threads(4), 'M': parpy.threads(64)}, opt_noalias_scopes=noalias))
     assert np.array_equal(ad.cpu().numpy(), wa) and np.array_equal(bd.cpu().numpy(), wb)
+
+
+def test_repeated_calls_take_the_short_path_and_stay_correct():
+    """A call whose argument signature and options were seen before goes straight to the launch plan;
+    anything that changes the specialisation (a scalar, a shape, an option, the alignment) must not."""
+    f = parpy.jit(K.axpy)
+    o = opts_for({'N': parpy.threads(256)})
+    x, y = torch.arange(1000, dtype=torch.float32, device="cuda"), torch.ones(1000, dtype=torch.float32, device="cuda")
+    out = torch.zeros(1000, dtype=torch.float32, device="cuda")
+    for rep in range(3):
+        out.zero_()
+        f(2.0, x, y, out, 1000, opts=o)
+        assert torch.equal(out, 2.0 * x + y)
+    assert len(f._seen_calls) >= 1
+    out2 = torch.zeros(1000, dtype=torch.float32, device="cuda")     # other buffers, same signature
+    f(2.0, y, x, out2, 1000, opts=o)
+    assert torch.equal(out2, 2.0 * y + x)
+    f(3.0, x, y, out, 1000, opts=o)                                   # another scalar: another specialisation
+    assert torch.equal(out, 3.0 * x + y)
+    o.parallelize = {'N': parpy.threads(64)}                          # options changed in place
+    f(3.0, x, y, out2, 1000, opts=o)
+    assert torch.equal(out2, 3.0 * x + y)
+    xs, ys, outs = x[:500], y[:500], torch.zeros(500, dtype=torch.float32, device="cuda")   # another shape
+    f(2.0, xs, ys, outs, 500, opts=o)
+    assert torch.equal(outs, 2.0 * xs + ys)
+    base = torch.arange(1001, dtype=torch.float32, device="cuda")
+    f(2.0, base[1:], y, out, 1000, opts=o)                            # a view that is only 4-byte aligned
+    f(2.0, base[1:], y, out, 1000, opts=o)
+    assert torch.equal(out, 2.0 * base[1:] + y)
+    with pytest.raises(RuntimeError, match="unsupported keyword arguments"):
+        f(2.0, x, y, out, 1000, opts=o, extra=1)
