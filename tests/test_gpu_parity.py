@@ -421,3 +421,55 @@ def test_repeated_calls_take_the_short_path_and_stay_correct():
     assert torch.equal(out, 2.0 * base[1:] + y)
     with pytest.raises(RuntimeError, match="unsupported keyword arguments"):
         f(2.0, x, y, out, 1000, opts=o, extra=1)
+
+
+def test_random_shapes_and_thread_counts():
+    """Row reductions, softmax and the element-wise copy over seeded random shapes and thread counts:
+    extents that do and do not divide by the vector width, the wavefront and the block size."""
+    rng = np.random.default_rng(2024)
+    for case in range(40):
+        N = int(rng.integers(1, 300))
+        M = int(rng.choice([1, 3, 4, 31, 64, 100, 127, 128, 255, 256, 1000, 1024, 1536, 4096, 5000]))
+        inner = int(rng.choice([0, 64, 100, 128, 256, 512, 1024, 2048]))
+        x = rng.uniform(-1, 1, (N, M)).astype(np.float32)
+        p = {'outer': parpy.threads(N)}
+        if inner:
+            p['inner'] = parpy.threads(inner)
+        fn = [K.sum_rows, K.max_rows, K.min_rows][case % 3]
+        out = np.zeros(N, dtype=np.float32)
+        parpy.jit(fn)(x, out, N, opts=opts_for(p))
+        want = {K.sum_rows: np.sum, K.max_rows: np.max, K.min_rows: np.min}[fn](x.astype(np.float64), axis=1)
+        assert np.allclose(out, want, atol=1e-4, rtol=1e-5), ("reduce", case, N, M, inner, fn.__name__)
+        if inner and inner <= 1024:
+            xd = torch.from_numpy(x).cuda()
+            od = torch.zeros_like(xd)
+            W.softmax(xd, N, M, od, opts=opts_for({'N': parpy.threads(N), 'M': parpy.threads(inner)}))
+            assert torch.allclose(od.cpu(), torch.softmax(torch.from_numpy(x), 1), atol=1e-5), ("softmax", case, N, M, inner)
+        n = N * M
+        threads = int(rng.choice([64, 256, 1000, 4096, max(64, n // 4), max(64, n // 16), n]))
+        tpb = int(rng.choice([64, 128, 256, 1024]))
+        flat = torch.from_numpy(x.reshape(-1).copy()).cuda()
+        dst = torch.zeros_like(flat)
+        W.copy_1d(flat, dst, opts=opts_for({'N': parpy.threads(threads).tpb(tpb)}))
+        assert torch.equal(dst, flat), ("copy", case, n, threads, tpb)
+
+
+def test_random_sddmm_and_hmm_configurations():
+    """Shapes on both sides of every pass's applicability conditions: inner dimensions that are / are not
+    multiples of 32 and 64 (lane groups, tiled transposition), few and many non-zeros, state counts
+    below and above one workgroup, odd thread counts."""
+    rng = np.random.default_rng(77)
+    for n, k, density in [(64, 8, 0.2), (100, 48, 0.1), (512, 96, 0.05), (640, 128, 0.02), (1000, 200, 0.01), (2048, 64, 0.01)]:
+        A, B, crows, cols, vals = W.make_sddmm(n, k, density, seed=int(rng.integers(1 << 30)))
+        rows = oracle.csr_rows(crows)
+        nnz = len(cols)
+        C = {"rows": torch.from_numpy(rows).cuda(), "cols": torch.from_numpy(cols).cuda(), "values": torch.from_numpy(vals).cuda(), "nnz": nnz}
+        D = torch.zeros(nnz, dtype=torch.float32, device="cuda")
+        W.sddmm_coo(torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda(), C, D, 0.5, -1.5, opts=opts_for({"nnz": parpy.threads(nnz).tpb(256)}))
+        want = oracle.sddmm(A, B, rows, cols, vals, alpha=0.5, beta=-1.5)
+        assert np.allclose(D.cpu().numpy(), want, atol=1e-4, rtol=1e-5), (n, k, density)
+    for k, threads, n_inst, max_len in [(2, 64, 3, 40), (3, 100, 5, 77), (4, 128, 7, 33), (5, 512, 4, 150), (6, 1024, 3, 60), (6, 2048, 2, 25)]:
+        hmm, seqs = W.synthetic_hmm(k, n_inst=n_inst, min_len=2, max_len=max_len, seed=int(rng.integers(1 << 30)))
+        got, _, _ = _run_synthetic(hmm, seqs, threads)
+        want = oracle.hmm_syn_forward(hmm, seqs, np.float32)
+        assert np.allclose(got, want, atol=1e-5, rtol=1e-5), (k, threads, n_inst, max_len, np.abs(got - want).max())
