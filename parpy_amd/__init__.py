@@ -49,7 +49,6 @@ def _convert_python_function_to_ir(fn, vars):
     filepath = inspect.getfile(fn)
     src, line_ofs, col_ofs = _get_source_code(fn)
     tree = python_ast.parse(src)
-    # a decorated function is parsed with its decorator lines: they do not belong to the body
     top_map = _get_tops(None)
     info = (filepath, line_ofs, col_ofs)
     # Names are resolved the way Python itself would for `fn` -- closure cells,
