@@ -31,12 +31,31 @@ def _is_cached(key):
     return os.path.isfile(_get_code_path(key))
 
 
+_pinned = set()  # keys of modules behind callables handed to the user (compile_string): never unloaded
+_plans = []     # (runtime library, plan handle) of every launch plan created, released by clear_cache
+
+
 def clear_cache():
-    """Remove every cached code object."""
+    """Remove every cached code object; release the launch plans (with the device temporaries they
+    keep) and the loaded modules once the device has finished what was enqueued."""
     import shutil
     shutil.rmtree(f"{cache_path}", ignore_errors=True)
     cache_path.mkdir(parents=True, exist_ok=True)
-    _modules.clear()
+    if _plans or _modules:
+        lib = _plans[0][0] if _plans else None
+        if lib is None:
+            from .runtime import load_hip_runtime_lib
+            lib = load_hip_runtime_lib()
+        if _plans:
+            lib.parpy_sync()
+        for l, plan in _plans:
+            l.parpy_hip_plan_destroy(plan)
+        for key, (module, _) in _modules.items():
+            if key not in _pinned:
+                lib.parpy_hip_module_unload(module)
+    _plans.clear()
+    for key in [k for k in _modules if k not in _pinned]:
+        del _modules[key]
 
 
 def hiprtc_compile(source, opts, lib=None):
@@ -111,6 +130,7 @@ def get_wrapper(name, key, plan_text, opts):
     if rc != 0:
         raise RuntimeError(lib.parpy_get_error_message().decode("ascii", "replace"))
 
+    _plans.append((lib, plan))
     if opts.use_cuda_graphs:
         lib.parpy_hip_plan_set_graph(plan, 1)
 
@@ -156,6 +176,7 @@ def get_string_wrapper(kernel_name, key, grid, block, opts):
     from .runtime import _compile_runtime_lib
     lib = _compile_runtime_lib(opts.backend)
     module = _load_module(key, lib)
+    _pinned.add(key)
     sizes = ScalarSizes(opts)
     g = (ctypes.c_int64 * 3)(*grid)
     b = (ctypes.c_int64 * 3)(*block)

@@ -473,3 +473,21 @@ def test_random_sddmm_and_hmm_configurations():
         got, _, _ = _run_synthetic(hmm, seqs, threads)
         want = oracle.hmm_syn_forward(hmm, seqs, np.float32)
         assert np.allclose(got, want, atol=1e-5, rtol=1e-5), (k, threads, n_inst, max_len, np.abs(got - want).max())
+
+
+def test_clear_cache_releases_and_recompiles():
+    f = parpy.jit(K.axpy)
+    o = opts_for({'N': parpy.threads(128)})
+    x, y = torch.arange(500, dtype=torch.float32, device="cuda"), torch.ones(500, dtype=torch.float32, device="cuda")
+    out = torch.zeros(500, dtype=torch.float32, device="cuda")
+    f(2.0, x, y, out, 500, opts=o)
+    src = 'extern "C" __global__ void twice(float* x, int n) { int i = blockIdx.x * blockDim.x + threadIdx.x; if (i < n) x[i] *= 2.0f; }'
+    g = parpy.compile_string("twice", src, opts_for({}), grid=(2, 1, 1), block=(256, 1, 1))
+    g(out, 500)
+    parpy.sync(HIP)
+    assert torch.equal(out, 2.0 * (2.0 * x + y))
+    parpy.clear_cache()                       # plans, their temporaries and modules go; files are removed
+    f(2.0, x, y, out, 500, opts=o)            # compiled again from scratch
+    g(out, 500)                               # a callable handed out earlier keeps working
+    parpy.sync(HIP)
+    assert torch.equal(out, 2.0 * (2.0 * x + y))
