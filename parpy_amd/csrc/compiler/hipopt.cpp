@@ -639,7 +639,7 @@ struct Pass {
             Interval r = expr_range(idx, env);
             if (!r.known || r.lo < 0 || r.hi >= numel) return e;  // the load is executed unconditionally once hoisted
             for (auto& h : hoisted)
-              if (h.load->args[0]->name == base && expr_eq(h.load->args[1], idx)) {
+              if (h.load->k == Expr::Index && h.load->args[0]->name == base && expr_eq(h.load->args[1], idx)) {
                 auto re = std::make_shared<Expr>();
                 re->k = Expr::RegElem;
                 re->ty = e->ty;
@@ -666,6 +666,88 @@ struct Pass {
           };
           Stmts nbody = rewrite_stmts(*is.body, try_hoist);
           if (hoisted.empty()) { out.push_back(s); continue; }
+          // Arithmetic whose operands are all hoisted values (or literals) is invariant too: `trans1[..] +
+          // trans2[..]` is computed once and takes one register per element instead of two.  Only values
+          // with a single use are combined, so the register count never grows; same operations in the
+          // same order, hence the same bits.
+          {
+            // `t = hoisted[slot]` is only a name for the value: uses of t become the register element
+            std::map<Name, E> alias;
+            visit_stmts(nbody, [&](const S& st) {
+              if (st->k == Stmt::Def && st->expr && st->expr->k == Expr::RegElem && !reassigned.count(st->id)) alias[st->id] = st->expr;
+            });
+            if (!alias.empty()) {
+              std::function<Stmts(const Stmts&)> drop = [&](const Stmts& b) {
+                Stmts o;
+                for (auto& c : b) {
+                  if (c->k == Stmt::Def && alias.count(c->id)) continue;
+                  auto n = clone(c);
+                  n->body = drop(c->body);
+                  n->els = drop(c->els);
+                  o.push_back(n);
+                }
+                return o;
+              };
+              nbody = rewrite_stmts(drop(nbody), [&](const E& x) -> E {
+                if (x->k != Expr::Var) return x;
+                auto it = alias.find(x->name);
+                return it == alias.end() ? x : it->second;
+              });
+            }
+          }
+          for (bool changed = true; changed;) {
+            changed = false;
+            std::map<Name, int> uses;
+            visit_stmts(nbody, [&](const S& st) {
+              auto scan = [&](const E& root) { visit_exprs(root, [&](const E& x) { if (x->k == Expr::RegElem) uses[x->name]++; }); };
+              scan(st->dst); scan(st->expr); scan(st->lo); scan(st->hi);
+            });
+            auto index_of = [&](const Name& r) { for (size_t q = 0; q < hoisted.size(); ++q) if (hoisted[q].reg == r) return (int)q; return -1; };
+            auto merge = [&](const E& e) -> E {
+              if (e->k != Expr::BinOpE || !e->ty.is_scalar() || elem_bytes(e->ty.sz) > 4) return e;
+              if (!(e->bop == BinOp::Add || e->bop == BinOp::Sub || e->bop == BinOp::Mul || e->bop == BinOp::Max || e->bop == BinOp::Min)) return e;
+              auto reg = [&](const E& x) { return x->k == Expr::RegElem && index_of(x->name) >= 0 && expr_eq(x->args[0], is.slot); };
+              auto lit = [](const E& x) { return x->k == Expr::Float || x->k == Expr::Int; };
+              const E &a = e->args[0], &b = e->args[1];
+              if (!((reg(a) && (reg(b) || lit(b))) || (lit(a) && reg(b)))) return e;
+              if (reg(a) && reg(b) && a->name == b->name) return e;
+              // the combined value takes the place of an operand that has no other use, so registers never grow
+              if (!((reg(a) && uses[a->name] == 1) || (reg(b) && uses[b->name] == 1))) return e;
+              Hoisted h;
+              E la = reg(a) ? hoisted[index_of(a->name)].load : a, lb = reg(b) ? hoisted[index_of(b->name)].load : b;
+              h.load = mk_binop(e->bop, la, lb, e->ty, e->i);
+              h.reg = gen.fresh("inv_expr");
+              h.sz = e->ty.sz;
+              if (reg(a)) uses[a->name]--;
+              if (reg(b)) uses[b->name]--;
+              hoisted.push_back(h);
+              uses[h.reg] = 1;
+              changed = true;
+              auto re = std::make_shared<Expr>();
+              re->k = Expr::RegElem;
+              re->ty = e->ty;
+              re->name = h.reg;
+              re->args = {is.slot};
+              return re;
+            };
+            nbody = rewrite_stmts(nbody, merge);
+          }
+          {
+            std::map<Name, int> uses;
+            visit_stmts(nbody, [&](const S& st) {
+              auto scan = [&](const E& root) { visit_exprs(root, [&](const E& x) { if (x->k == Expr::RegElem) uses[x->name]++; }); };
+              scan(st->dst); scan(st->expr); scan(st->lo); scan(st->hi);
+            });
+            std::vector<Hoisted> live;
+            for (auto& h : hoisted) {
+              int64_t cost = is.slots * std::max(1, elem_bytes(h.sz) / 4);
+              if (uses[h.reg] > 0) live.push_back(h);
+              else if (h.load->k == Expr::Index) *budget += cost;   // a load that only feeds a combined value
+            }
+            for (auto& h : live)
+              if (h.load->k != Expr::Index) *budget -= is.slots * std::max(1, elem_bytes(h.sz) / 4);
+            hoisted = live;
+          }
           // loop nest that fills the registers, with the same thread mapping
           std::map<Name, Name> ren;
           Name nq = gen.fresh(s->id.s);
@@ -702,9 +784,12 @@ struct Pass {
             re->ty = Type::scalar(h.sz);
             re->name = h.reg;
             re->args = {fill_slot};
-            auto ld = std::make_shared<Expr>(*h.load);
-            ld->args = {h.load->args[0], subst_vars(h.load->args[1], rv)};
-            ld->dim_idx.clear();
+            E ld = rewrite_expr(subst_vars(h.load, rv), [](const E& x) -> E {
+              if (x->k != Expr::Index || x->dim_idx.empty()) return x;
+              auto c = std::make_shared<Expr>(*x);
+              c->dim_idx.clear();
+              return c;
+            });
             fills.push_back(mk_assign(re, ld));
           }
           if (is.inner) {
