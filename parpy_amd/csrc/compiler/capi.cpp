@@ -1,5 +1,6 @@
 // C ABI of the compiler core (declared in include/parpy_hipc.h).
 #include <cstring>
+#include <chrono>
 #include <sstream>
 
 #include "../../../include/parpy_hipc.h"
@@ -77,8 +78,12 @@ int32_t parpy_hipc_compile(const parpy_hipc_fun* f, const char* args, const char
     Options opts = parse_options(opts_text);
     NameGen gen = f->pf->gen;  // the parsed function is shared: every compilation numbers its names from the same start
     std::ostringstream dbg;
+    // every dump carries the time since the start of the compilation (src/utils/debug.rs:10-37)
+    auto t0 = std::chrono::steady_clock::now();
     auto stage = [&](const char* name, const std::string& text) {
-      if (opts.debug_print) dbg << "=== " << name << " ===\n" << text << "\n";
+      if (!opts.debug_print) return;
+      auto us = std::chrono::duration_cast<std::chrono::microseconds>(std::chrono::steady_clock::now() - t0).count();
+      dbg << "=== " << name << " (time: " << us << " us) ===\n" << text << "\n";
     };
     FunDef spec = specialize(*f->pf, a, opts, gen);
     stage("specialised and type-checked", print_fun(spec));
