@@ -78,10 +78,14 @@ template <int CTRL, class T> __device__ __forceinline__ T parpy_dpp(T v) {
     int x = __builtin_bit_cast(int, v);
     x = __builtin_amdgcn_update_dpp(x, x, CTRL, 0xF, 0xF, false);
     return __builtin_bit_cast(T, x);
-  } else {
-    int x = (int)v;
+  } else if constexpr (sizeof(T) == 2) {   // the bits travel, not the value: a half must not be rounded to an integer
+    int x = (int)__builtin_bit_cast(unsigned short, v);
     x = __builtin_amdgcn_update_dpp(x, x, CTRL, 0xF, 0xF, false);
-    return (T)x;
+    return __builtin_bit_cast(T, (unsigned short)x);
+  } else {
+    int x = (int)__builtin_bit_cast(unsigned char, v);
+    x = __builtin_amdgcn_update_dpp(x, x, CTRL, 0xF, 0xF, false);
+    return __builtin_bit_cast(T, (unsigned char)x);
   }
 }
 template <class T> __device__ __forceinline__ T parpy_readlane(T v, int lane) {
@@ -93,8 +97,10 @@ template <class T> __device__ __forceinline__ T parpy_readlane(T v, int lane) {
     return __builtin_bit_cast(T, x);
   } else if constexpr (sizeof(T) == 4) {
     return __builtin_bit_cast(T, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+  } else if constexpr (sizeof(T) == 2) {
+    return __builtin_bit_cast(T, (unsigned short)__builtin_amdgcn_readlane((int)__builtin_bit_cast(unsigned short, v), lane));
   } else {
-    return (T)__builtin_amdgcn_readlane((int)v, lane);
+    return __builtin_bit_cast(T, (unsigned char)__builtin_amdgcn_readlane((int)__builtin_bit_cast(unsigned char, v), lane));
   }
 }
 struct parpy_op_add { template <class T> __device__ __forceinline__ T operator()(T a, T b) const { return a + b; } };

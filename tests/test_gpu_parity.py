@@ -491,3 +491,26 @@ def test_clear_cache_releases_and_recompiles():
     g(out, 500)                               # a callable handed out earlier keeps working
     parpy.sync(HIP)
     assert torch.equal(out, 2.0 * (2.0 * x + y))
+
+
+@pytest.mark.parametrize("dtype", [np.float64, np.float16, np.int32, np.int64, np.int16, np.uint32], ids=lambda d: np.dtype(d).name)
+def test_reductions_over_element_types(dtype):
+    """Wavefront and workgroup reductions for 2-, 4- and 8-byte elements (the cross-lane steps move
+    64-bit values as two halves and widen 16-bit ones), in one wavefront, one workgroup and several."""
+    rng = np.random.default_rng(5)
+    N = 37
+    for M, inner in [(50, 64), (700, 256), (3000, 2048)]:
+        if np.issubdtype(dtype, np.floating):
+            x = rng.uniform(0.5, 1.5, (N, M)).astype(dtype)
+        else:
+            x = rng.integers(1, 4, (N, M)).astype(dtype)
+        for fn, ref in [(K.sum_rows, np.sum), (K.max_rows, np.max), (K.min_rows, np.min)]:
+            out = np.zeros(N, dtype=dtype)
+            parpy.jit(fn)(x, out, N, opts=opts_for({'outer': parpy.threads(N), 'inner': parpy.threads(inner)}))
+            want = ref(x.astype(np.float64), axis=1)
+            if dtype == np.float16:
+                assert np.allclose(out.astype(np.float64), want, rtol=2e-2), (fn.__name__, M, inner)
+            elif np.issubdtype(dtype, np.floating):
+                assert np.allclose(out, want, rtol=1e-12), (fn.__name__, M, inner)
+            else:
+                assert np.array_equal(out.astype(np.int64), want.astype(np.int64)), (fn.__name__, M, inner)
