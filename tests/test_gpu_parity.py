@@ -514,3 +514,37 @@ def test_reductions_over_element_types(dtype):
                 assert np.allclose(out, want, rtol=1e-12), (fn.__name__, M, inner)
             else:
                 assert np.array_equal(out.astype(np.int64), want.astype(np.int64)), (fn.__name__, M, inner)
+
+
+@pytest.mark.parametrize("dtype", [torch.float64, torch.float16, torch.int32, torch.int8], ids=lambda d: str(d).split(".")[1])
+def test_elementwise_and_softmax_over_element_types(dtype):
+    """Vectorised element-wise loops with 8-, 4-, 2- and 1-byte elements; softmax in double and half."""
+    for n, threads, tpb in [(4096, 256, 64), (1 << 16, 1 << 12, 256), (1000, 1000, 128)]:
+        x = (torch.arange(n, device="cuda") % 100).to(dtype)
+        out = torch.zeros_like(x)
+        W.copy_1d(x, out, opts=opts_for({'N': parpy.threads(threads).tpb(tpb)}))
+        assert torch.equal(out, x), (n, threads, tpb)
+    if dtype.is_floating_point:
+        N, M = 64, 512
+        x = torch.randn((N, M), dtype=torch.float64).to(dtype)
+        xd = x.cuda()
+        od = torch.zeros_like(xd)
+        W.softmax(xd, N, M, od, opts=opts_for({'N': parpy.threads(N), 'M': parpy.threads(128)}))
+        want = torch.softmax(x.double(), 1)
+        assert torch.allclose(od.cpu().double(), want, atol=2e-3 if dtype == torch.float16 else 1e-12)
+
+
+@pytest.mark.parametrize("k,threads", [(4, 128), (5, 1024), (6, 1024)])
+def test_forward_in_double_precision(k, threads):
+    """The same kernel on float64 tables and state vectors (8-byte LDS rows, two-element vectors,
+    64-bit cross-lane moves) against the fp64 oracle: agreement to double rounding."""
+    hmm, seqs = W.synthetic_hmm(k, n_inst=6, min_len=30, max_len=200)
+    hmm64 = {key: (v.astype(np.float64) if isinstance(v, np.ndarray) and v.dtype == np.float32 else v) for key, v in hmm.items()}
+    hd, sd = W.to_device(hmm64), W.to_device(seqs)
+    n, S = seqs["num_instances"], hmm["num_states"]
+    a1 = torch.zeros((n, S), dtype=torch.float64, device="cuda")
+    a2 = torch.zeros_like(a1)
+    res = torch.zeros(n, dtype=torch.float64, device="cuda")
+    W.forward_syn(hd, sd, res, a1, a2, opts=opts_for({'inst': parpy.threads(n), 'state': parpy.threads(threads)}))
+    want = oracle.hmm_syn_forward(hmm, seqs, np.float64)
+    assert np.allclose(res.cpu().numpy(), want, atol=0, rtol=1e-12), np.abs(res.cpu().numpy() - want).max()
