@@ -222,7 +222,7 @@ struct DevicePrinter {
     if (!opts.opt_narrow_index || !is_i64(e)) { r.s = pexpr_plain(e); return r; }
     switch (e->k) {
       case Expr::Int:
-        if (e->iv >= INT32_MIN && e->iv <= INT32_MAX) { r.s = std::to_string(e->iv); r.narrow = true; }
+        if (e->iv >= INT32_MIN && e->iv <= INT32_MAX) { r.s = e->iv < 0 ? "(" + std::to_string(e->iv) + ")" : std::to_string(e->iv); r.narrow = true; }
         else r.s = "((int64_t)" + std::to_string(e->iv) + "LL)";
         return r;
       case Expr::Var: {
@@ -319,12 +319,15 @@ struct DevicePrinter {
           return "((int64_t)" + std::to_string(e->iv) + "LL)";
         }
         if (e->ty.is_scalar() && e->ty.sz != ElemSize::I32) return "((" + std::string(elem_ctype(e->ty.sz)) + ")" + std::to_string(e->iv) + ")";
-        return std::to_string(e->iv);
+        return e->iv < 0 ? "(" + std::to_string(e->iv) + ")" : std::to_string(e->iv);
       }
-      case Expr::Float:
-        if (e->ty.sz == ElemSize::F64) return fmt_f64(e->fv);
+      case Expr::Float: {
+        // negative literals are parenthesised: `-` in front of one must not read as a decrement
+        bool neg = std::signbit(e->fv) && !std::isnan(e->fv) && !std::isinf(e->fv);
+        if (e->ty.sz == ElemSize::F64) return neg ? "(" + fmt_f64(e->fv) + ")" : fmt_f64(e->fv);
         if (e->ty.sz == ElemSize::F16) return "((_Float16)" + fmt_f32(e->fv) + ")";
-        return fmt_f32(e->fv);
+        return neg ? "(" + fmt_f32(e->fv) + ")" : fmt_f32(e->fv);
+      }
       case Expr::Bool: return e->bv ? "true" : "false";
       case Expr::UnOpE: {
         std::string a = pexpr(e->args[0]);
@@ -335,7 +338,7 @@ struct DevicePrinter {
           return fn + paren(a);
         };
         switch (e->uop) {
-          case UnOp::Sub: return "(-" + a + ")";
+          case UnOp::Sub: return "(-" + paren(a) + ")";
           case UnOp::Not: return "(!" + a + ")";
           case UnOp::BitNeg: return "(~" + a + ")";
           // single precision: the hardware base-2 instructions with the scale folded in

@@ -418,3 +418,54 @@ def test_entry_function_rules():
             x[:] += y[:]
     with pytest.raises(RuntimeError, match="Missing required keyword argument opts in call to fun_with_args"):
         fun_with_args(np.ndarray((10,), dtype=np.float32), np.ndarray((10,), dtype=np.float32))
+
+
+# ---------------------------------------------------------------- random expression trees: device against the interpreter
+def _random_expr(rng, depth, kind):
+    # `//` and `%` get non-negative operands: they compile to C's truncating operators, which agree
+    # with Python's flooring ones only there (src/cuda/pprint.rs:146-147 of the reference does the same)
+    leaves = ["a[i]", "b[i]", "c[i]"] + (["0.5", "2.0", "1.25"] if kind == "f" else ["3", "7", "2"])
+    if depth == 0 or rng.random() < 0.2:
+        return str(rng.choice(leaves))
+    x, y = _random_expr(rng, depth - 1, kind), _random_expr(rng, depth - 1, kind)
+    if kind == "f":
+        forms = ["({x} + {y})", "({x} - {y})", "({x} * {y})", "({x} / (abs({y}) + 1.0))", "ops.max({x}, {y})", "ops.min({x}, {y})",
+                 "abs({x})", "(-{x})", "ops.exp(ops.min({x}, 2.0))", "ops.sqrt(abs({x}))", "({x} if {x} < {y} else {y})",
+                 "ops.tanh({x})", "ops.log(abs({x}) + 1.0)"]
+    else:
+        forms = ["({x} + {y})", "({x} - {y})", "({x} * {y})", "(abs({x}) // (abs({y}) + 1))", "(abs({x}) % (abs({y}) + 1))", "({x} & {y})",
+                 "({x} | {y})", "({x} ^ {y})", "ops.max({x}, {y})", "ops.min({x}, {y})", "abs({x})", "(-{x})",
+                 "({x} if {x} <= {y} else {y})", "(({x} & 7) << 2)", "(abs({x}) >> 1)"]
+    return str(rng.choice(forms)).format(x=x, y=y)
+
+
+def _loop_fun(name, expr):
+    src = f"def {name}(out, a, b, c, N):\n    parpy.label('N')\n    for i in range(N):\n        out[i] = {expr}\n"
+    fname = f"<{name}>"
+    linecache.cache[fname] = (len(src), None, src.splitlines(True), fname)
+    ns = {"parpy": parpy, "ops": ops}
+    exec(compile(src, fname, "exec"), ns)
+    return ns[name]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind,dtype", [("f", np.float32), ("f", np.float64), ("i", np.int32), ("i", np.int64)], ids=["f32", "f64", "i32", "i64"])
+def test_random_expressions_on_device(kind, dtype):
+    rng = np.random.default_rng(31)
+    N = 96
+    for case in range(25):
+        expr = _random_expr(rng, 4, kind)
+        f = _loop_fun(f"expr_{kind}_{case}", expr)
+        if kind == "f":
+            args = [rng.uniform(-2, 2, N).astype(dtype) for _ in range(3)]
+        else:
+            args = [rng.integers(-20, 20, N).astype(dtype) for _ in range(3)]
+        want, got = np.zeros(N, dtype=dtype), np.zeros(N, dtype=dtype)
+        with np.errstate(all="ignore"):
+            f(want, *args, N)
+        parpy.jit(f)(got, *args, N, opts=opts_for({'N': parpy.threads(N)}))
+        if kind == "f":
+            ok = np.allclose(got, want, rtol=2e-5 if dtype == np.float32 else 1e-12, atol=1e-6 if dtype == np.float32 else 1e-13, equal_nan=True)
+        else:
+            ok = np.array_equal(got, want)
+        assert ok, (expr, got[:4], want[:4])
