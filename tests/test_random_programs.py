@@ -1,0 +1,115 @@
+"""Seeded random loop nests -- row reductions with post-processing, element-wise 2-D updates, two-phase
+row normalisations and time loops over ping-pong buffers -- compiled under several parallelisations and
+compared with the Python interpreter running the very same function (the reference's own test method,
+e.g. test/test_slicing.py:111-115)."""
+import linecache
+
+import numpy as np
+import pytest
+
+import parpy_amd as parpy
+import parpy_amd.operators as ops
+from parpy_amd.compile import hiprtc_compile
+
+HIP = parpy.CompileBackend.Hip
+
+
+def opts_for(p):
+    o = parpy.par(p)
+    o.backend = HIP
+    return o
+
+
+def build(name, src):
+    fname = f"<{name}>"
+    linecache.cache[fname] = (len(src), None, src.splitlines(True), fname)
+    ns = {"parpy": parpy, "ops": ops}
+    exec(compile(src, fname, "exec"), ns)
+    return ns[name]
+
+
+def term(rng):
+    return str(rng.choice(["x[i, j]", "y[j]", "(x[i, j] * y[j])", "(x[i, j] + z[i])", "abs(x[i, j])", "(x[i, j] - 0.5)",
+                           "ops.max(x[i, j], y[j])", "(x[i, j] * x[i, j])", "ops.exp(ops.min(x[i, j], 1.0))"]))
+
+
+def make_program(rng, case):
+    kind = case % 4
+    name = f"prog_{case}"
+    if kind == 0:      # row reduction, then something with the result
+        op = str(rng.choice(["+", "max", "min"]))
+        init = {"+": "0.0", "max": "-ops.inf", "min": "ops.inf"}[op]
+        upd = f"acc + {term(rng)}" if op == "+" else f"ops.{op}(acc, {term(rng)})"
+        post = str(rng.choice(["acc", "(acc * z[i])", "(acc if acc > z[i] else z[i])", "ops.sqrt(abs(acc))", "(acc + 1.0)"]))
+        src = (f"def {name}(x, y, z, out, out2, N, M):\n    parpy.label('outer')\n    for i in range(N):\n"
+               f"        acc = ops.float32({init})\n        parpy.label('inner')\n        for j in range(M):\n            acc = {upd}\n"
+               f"        out[i] = {post}\n")
+    elif kind == 1:    # element-wise 2-D update
+        src = (f"def {name}(x, y, z, out, out2, N, M):\n    parpy.label('outer')\n    for i in range(N):\n"
+               f"        parpy.label('inner')\n        for j in range(M):\n            out2[i, j] = {term(rng)} + {term(rng)}\n")
+    elif kind == 2:    # two phases over the row with a reduction in between
+        red = str(rng.choice(["max", "sum"]))
+        use = str(rng.choice(["x[i, :] - m", "x[i, :] * m", "ops.max(x[i, :], m)"]))
+        src = (f"def {name}(x, y, z, out, out2, N, M):\n    parpy.label('outer')\n    for i in range(N):\n"
+               f"        parpy.label('inner')\n        m = ops.{red}(x[i, :])\n        parpy.label('inner')\n        out2[i, :] = {use}\n"
+               f"        parpy.label('inner')\n        out[i] = ops.sum(out2[i, :])\n")
+    else:              # time loop over two buffers selected by parity, inner loop parallel
+        steps = int(rng.integers(2, 6))
+        mix = str(rng.choice(["0.5 * (src[i, j] + src[i, (j + 1) % M])", "ops.max(src[i, j], src[i, (j + M - 1) % M]) - 0.25",
+                              "src[i, j] * y[j] + z[i]"]))
+        src = (f"def {name}(x, y, z, out, out2, N, M):\n    parpy.label('outer')\n    for i in range(N):\n"
+               f"        for t in range({steps}):\n            src = x\n            dst = out2\n            if t & 1:\n"
+               f"                src = out2\n                dst = x\n            parpy.label('inner')\n            for j in range(M):\n"
+               f"                dst[i, j] = {mix}\n        parpy.label('inner')\n        s1 = ops.sum(x[i, :])\n"
+               f"        parpy.label('inner')\n        s2 = ops.sum(out2[i, :])\n        out[i] = s1 + s2\n")
+    return name, src, kind
+
+
+def par_specs(kind, N, M):
+    specs = [{'outer': parpy.threads(N)}]
+    for inner in (64, 256):
+        p = parpy.threads(inner)
+        specs.append({'outer': parpy.threads(N), 'inner': p.reduce() if kind == 0 else p})
+    if kind in (0, 1):
+        p = parpy.threads(2048)
+        specs.append({'outer': parpy.threads(N), 'inner': p.reduce() if kind == 0 else p})
+    return specs
+
+
+def inputs(rng, N, M):
+    x = rng.uniform(-1, 1, (N, M)).astype(np.float32)
+    y = rng.uniform(-1, 1, M).astype(np.float32)
+    z = rng.uniform(-1, 1, N).astype(np.float32)
+    return x, y, z, np.zeros(N, dtype=np.float32), np.zeros((N, M), dtype=np.float32)
+
+
+CASES = list(range(32))
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_random_programs_compile(case):
+    rng = np.random.default_rng(1000 + case)
+    name, src, kind = make_program(rng, case)
+    f = build(name, src)
+    N, M = 7, 96
+    for p in par_specs(kind, N, M)[:2]:
+        s = parpy.print_compiled(f, list(inputs(rng, N, M)) + [N, M], opts_for(p))
+        hiprtc_compile(s[:s.index("// host side")], opts_for({}))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", CASES)
+def test_random_programs_on_device(case):
+    rng = np.random.default_rng(1000 + case)
+    name, src, kind = make_program(rng, case)
+    f = build(name, src)
+    for N, M in [(5, 64), (9, 200), (3, 2048)]:
+        base = inputs(rng, N, M)
+        want = [a.copy() for a in base]
+        with np.errstate(all="ignore"):
+            f(*want, N, M)
+        for p in par_specs(kind, N, M):
+            got = [a.copy() for a in base]
+            parpy.jit(f)(*got, N, M, opts=opts_for(p))
+            for g, w, label in zip(got, want, "xyz oO"):
+                assert np.allclose(g, w, rtol=1e-4, atol=1e-4, equal_nan=True), (src, N, M, sorted(p), label, np.abs(g - w).max())
