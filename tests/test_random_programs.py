@@ -86,6 +86,76 @@ def inputs(rng, N, M):
 CASES = list(range(32))
 
 
+# ---------------------------------------------------------------- further shapes
+def more_program(rng, case):
+    kind = case % 4
+    name = f"more_{case}"
+    if kind == 0:      # three levels: rows, columns, a reduction over a third dimension
+        upd = str(rng.choice(["acc + w[i, j, k] * v[k]", "ops.max(acc, w[i, j, k] + v[k])", "acc + abs(w[i, j, k] - v[k])"]))
+        init = "-ops.inf" if "max" in upd else "0.0"
+        src = (f"def {name}(w, v, x, idx, out2, N, M, K):\n    parpy.label('outer')\n    for i in range(N):\n"
+               f"        parpy.label('mid')\n        for j in range(M):\n            acc = ops.float32({init})\n"
+               f"            parpy.label('inner')\n            for k in range(K):\n                acc = {upd}\n            out2[i, j] = acc\n")
+    elif kind == 1:    # data-dependent while loop per element (integer work)
+        src = (f"def {name}(w, v, x, idx, out2, N, M, K):\n    parpy.label('outer')\n    for i in range(N):\n"
+               f"        parpy.label('mid')\n        for j in range(M):\n            n = idx[j] + i + 1\n            c = 0\n"
+               f"            while n != 1 and c < 50:\n                if n % 2 == 0:\n                    n = n // 2\n"
+               f"                else:\n                    n = 3 * n + 1\n                c = c + 1\n            out2[i, j] = ops.float32(c)\n")
+    elif kind == 2:    # a branch on a per-row value with the same parallel structure on both sides
+        a, b = str(rng.choice(["x[i, j] * 2.0", "x[i, j] + v[0]", "abs(x[i, j])"])), str(rng.choice(["-x[i, j]", "x[i, j] * x[i, j]", "0.25"]))
+        src = (f"def {name}(w, v, x, idx, out2, N, M, K):\n    parpy.label('outer')\n    for i in range(N):\n"
+               f"        if x[i, 0] > 0.0:\n            parpy.label('mid')\n            for j in range(M):\n                out2[i, j] = {a}\n"
+               f"        else:\n            parpy.label('mid')\n            for j in range(M):\n                out2[i, j] = {b}\n")
+    else:              # gather through an index array
+        src = (f"def {name}(w, v, x, idx, out2, N, M, K):\n    parpy.label('outer')\n    for i in range(N):\n"
+               f"        parpy.label('mid')\n        for j in range(M):\n            out2[i, j] = x[i, idx[j]] + x[(i + 1) % N, idx[(j + 3) % M]]\n")
+    return name, src, kind
+
+
+MORE = list(range(12))
+
+
+def more_inputs(rng, N, M, K):
+    return (rng.uniform(-1, 1, (N, M, K)).astype(np.float32), rng.uniform(-1, 1, K).astype(np.float32),
+            rng.uniform(-1, 1, (N, M)).astype(np.float32), rng.permutation(M).astype(np.int64), np.zeros((N, M), dtype=np.float32))
+
+
+def more_specs(kind, N, M):
+    specs = [{'outer': parpy.threads(N)}, {'outer': parpy.threads(N), 'mid': parpy.threads(M)}, {'outer': parpy.threads(N), 'mid': parpy.threads(64)}]
+    if kind == 0:
+        specs += [{'outer': parpy.threads(N), 'mid': parpy.threads(M), 'inner': parpy.threads(64).reduce()},
+                  {'outer': parpy.threads(N), 'inner': parpy.threads(128).reduce()}]
+    return specs
+
+
+@pytest.mark.parametrize("case", MORE)
+def test_more_random_programs_compile(case):
+    rng = np.random.default_rng(2000 + case)
+    name, src, kind = more_program(rng, case)
+    f = build(name, src)
+    N, M, K = 4, 24, 40
+    for p in more_specs(kind, N, M):
+        s = parpy.print_compiled(f, list(more_inputs(rng, N, M, K)) + [N, M, K], opts_for(p))
+        hiprtc_compile(s[:s.index("// host side")], opts_for({}))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", MORE)
+def test_more_random_programs_on_device(case):
+    rng = np.random.default_rng(2000 + case)
+    name, src, kind = more_program(rng, case)
+    f = build(name, src)
+    for N, M, K in [(4, 24, 40), (3, 130, 70)]:
+        base = more_inputs(rng, N, M, K)
+        want = [a.copy() for a in base]
+        with np.errstate(all="ignore"):
+            f(*want, N, M, K)
+        for p in more_specs(kind, N, M):
+            got = [a.copy() for a in base]
+            parpy.jit(f)(*got, N, M, K, opts=opts_for(p))
+            assert np.allclose(got[-1], want[-1], rtol=1e-4, atol=1e-4), (src, N, M, K, sorted(p), np.abs(got[-1] - want[-1]).max())
+
+
 @pytest.mark.parametrize("case", CASES)
 def test_random_programs_compile(case):
     rng = np.random.default_rng(1000 + case)
