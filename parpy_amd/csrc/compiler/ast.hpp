@@ -376,6 +376,7 @@ struct Options {  // src/option.rs:14-108
   bool opt_unswitch = false;   // measured slower on the HMM kernels (higher register pressure): opt-in
   bool opt_gather_transpose = true;
   bool opt_noalias_scopes = false; // aliases that always name different arrays are declared not to alias; measured slower on the HMM kernels: opt-in
+  bool opt_drop_barriers = true;   // barriers between regions that share no written array are removed
   bool opt_lane_split = true;      // eight lanes share each long per-thread dot product
   bool opt_nontemporal = true;   // non-temporal stores to arrays a kernel only writes
   int64_t reg_budget = 0;     // 32-bit registers per thread the caching passes may claim (0 = by block size)

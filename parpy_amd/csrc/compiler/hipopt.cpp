@@ -1032,6 +1032,92 @@ struct Pass {
     k.body = {nr};
   }
 
+  // ================================================================ barriers that order nothing
+  // The generic pipeline puts a barrier after every parallel loop.  Once rows live in registers, a
+  // loop may touch no memory at all (softmax's `exp` and scaling steps), and the barrier after it --
+  // or the one before the next memory access -- orders nothing.  A barrier between two straight-line
+  // regions of the workgroup's top-level statement list is kept only if an array written on one
+  // side is accessed on the other; accesses through pointer variables, helper calls and raw
+  // statements count as touching everything.  Barriers inside sequential loops are left alone (the
+  // region after them wraps round to the loop head).  Reduction sites own their LDS slots and
+  // synchronise internally.
+  struct Touched {
+    std::set<Name> r, w;
+    bool any = false;
+  };
+
+  void touched(const Stmts& ss, const std::set<Name>& arrays, Touched& t) {
+    std::function<void(const E&, bool)> scan = [&](const E& e, bool store) {
+      if (!e) return;
+      if (e->k == Expr::Index || e->k == Expr::AddrOf) {
+        const E& b = e->args[0];
+        if (b->k == Expr::Var && arrays.count(b->name)) (store && e->k == Expr::Index ? t.w : t.r).insert(b->name);
+        else t.any = true;
+        if (e->k == Expr::AddrOf) t.any = true;   // the address escapes (an external may write through it)
+        scan(e->args[1], false);
+        return;
+      }
+      if (e->k == Expr::Call) t.any = true;
+      for (auto& a : e->args) scan(a, false);
+    };
+    for (auto& st : ss) {
+      if (st->k == Stmt::RawStmt || st->k == Stmt::CallStmt) t.any = true;
+      scan(st->dst, st->k == Stmt::Assign);
+      scan(st->expr, false);
+      scan(st->lo, false);
+      scan(st->hi, false);
+      for (auto& a : st->args) scan(a, false);
+      touched(st->body, arrays, t);
+      touched(st->els, arrays, t);
+    }
+  }
+
+  Stmts drop_barriers_in(const Stmts& ss, const std::set<Name>& arrays) {
+    // split into regions at the barriers of this level
+    std::vector<Stmts> regions(1);
+    for (auto& st : ss) {
+      if (st->k == Stmt::Sync) regions.emplace_back();
+      else regions.back().push_back(st);
+    }
+    if (regions.size() == 1) {
+      Stmts out;
+      for (auto& st : ss) {
+        if (st->k == Stmt::For && st->map.k == GpuMap::Block) {  // the workgroup's statement list is further in
+          auto r = clone(st);
+          r->body = drop_barriers_in(st->body, arrays);
+          out.push_back(r);
+        } else out.push_back(st);
+      }
+      return out;
+    }
+    Stmts out = regions[0];
+    Touched before;
+    touched(regions[0], arrays, before);
+    for (size_t q = 1; q < regions.size(); ++q) {
+      Touched after;
+      touched(regions[q], arrays, after);
+      bool conflict = before.any || after.any;
+      for (auto& n : before.w) if (after.r.count(n) || after.w.count(n)) conflict = true;
+      for (auto& n : before.r) if (after.w.count(n)) conflict = true;
+      if (conflict) {
+        out.push_back(mk_sync());
+        before = after;
+      } else {   // merged into one region
+        before.r.insert(after.r.begin(), after.r.end());
+        before.w.insert(after.w.begin(), after.w.end());
+      }
+      for (auto& st : regions[q]) out.push_back(st);
+    }
+    return out;
+  }
+
+  void drop_barriers() {
+    std::set<Name> arrays;
+    for (auto& p : k.params) if (p.ty.is_pointer()) arrays.insert(p.id);
+    visit_stmts(k.body, [&](const S& st) { if (st->k == Stmt::LdsDecl) arrays.insert(st->id); });
+    k.body = drop_barriers_in(k.body, arrays);
+  }
+
   // ================================================================ no-alias scopes for array aliases
   // `src = a; dst = b; if (c) { src = b; dst = a; } <rest>`: in <rest> the two aliases always name
   // different arrays, but the target compiler only sees two selected pointers that may be equal, so
@@ -1612,6 +1698,7 @@ void hip_optimize(Program& p, const Options& opts, NameGen& gen) {
     int64_t budget = pass.reg_budget();
     if (opts.opt_hoist_invariant) k.body = pass.hoist_invariant(k.body, &budget, false);
     if (opts.opt_reg_cache) pass.reg_cache(&budget);
+    if (opts.opt_drop_barriers) pass.drop_barriers();
     if (opts.opt_noalias_scopes) k.body = pass.noalias_scopes(k.body);
     pass.mark_read_only();
     k.aligned_params = opts.assume_aligned;

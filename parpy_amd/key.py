@@ -42,6 +42,6 @@ def _ast_key(ir_ast):
 def _generate_fast_cache_key(ir_ast, args, opts):
     extra = [getattr(opts, n, None) for n in ("opt_vectorize", "opt_lds_rows", "opt_reg_cache",
                                               "opt_hoist_invariant", "opt_narrow_index", "opt_mfma_sddmm",
-                                              "opt_unswitch", "opt_gather_transpose", "opt_nontemporal", "opt_lane_split", "opt_noalias_scopes", "assume_aligned", "reg_budget")]
+                                              "opt_unswitch", "opt_gather_transpose", "opt_nontemporal", "opt_lane_split", "opt_drop_barriers", "opt_noalias_scopes", "assume_aligned", "reg_budget")]
     # a tuple: the (long) printed function keeps its cached hash from one call to the next
     return (_ast_key(ir_ast), _print_arguments_key(args), str(opts), tuple(extra))

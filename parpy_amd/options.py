@@ -242,6 +242,7 @@ class CompileOptions:
         self.opt_gather_transpose = None
         self.opt_nontemporal = None
         self.opt_lane_split = None
+        self.opt_drop_barriers = None
         self.opt_noalias_scopes = None
         self.reg_budget = None       # registers per thread the caching passes may claim (None: by block size)
         self.assume_aligned = None   # set by the driver: False when an array argument is not 16-byte aligned
