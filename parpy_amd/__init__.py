@@ -278,7 +278,7 @@ def jit(fun):
                 if hit is not None:
                     return hit.run_pointers(call[1])
         else:
-            call = None
+            call = key = None
         opts = backend._resolve_backend(_check_kwargs(kwargs, fun.__name__), True)
         checked = check_arguments(args, opts, True)
         wrap_fn = _compile_function(ir_ast, checked, opts)
@@ -286,7 +286,10 @@ def jit(fun):
         if call is not None and getattr(wrap_fn, "run_pointers", None) is not None:
             if len(seen) > 256:
                 seen.clear()
-            seen[(call[0], call[2], opts._fast_key())] = wrap_fn   # (backend resolution may have touched opts)
+            # under the state the caller passed (a fresh object with equal settings finds it) and
+            # under the state after backend resolution (the same object passed again finds it)
+            seen[key] = wrap_fn
+            seen[(call[0], call[2], opts._fast_key())] = wrap_fn
     _ir_asts[inner] = ir_ast
     inner._seen_calls = seen
     return inner

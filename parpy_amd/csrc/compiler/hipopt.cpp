@@ -501,7 +501,10 @@ struct Pass {
         int V = vector_width(s);
         bool nested = false;
         visit_stmts(s->body, [&](const S& c) { if (c->k == Stmt::For && c->map.k != GpuMap::None) nested = true; });
-        if (V > 0 && !nested && extent > 0 && extent % (s->map.n * V) == 0) {
+        // a block-level loop only needs whole vectors (threads may run different trip counts); a grid-wide
+        // one must also fill its launch exactly, since it has no bounds guard
+        // (fewer vectors than threads would leave threads idle that the scalar loop keeps busy)
+        if (V > 0 && !nested && extent >= s->map.n * V && extent % V == 0 && (!grid_wide || extent % (s->map.n * V) == 0)) {
           Type ity = Type::scalar(isz);
           Name q = gen.fresh(s->id.s + "_q"), u = gen.fresh(s->id.s + "_u");
           E d = fold_expr(mk_binop(BinOp::Add, s->lo,

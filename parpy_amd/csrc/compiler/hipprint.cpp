@@ -524,6 +524,17 @@ struct DevicePrinter {
     }
     std::string cond = v + cmp + his;
     if (!guard.empty()) cond += " && " + guard;
+    {
+      // a strided loop whose trip count differs per thread is not unrolled by the compiler on its own; with one
+      // iteration at a time every thread has a single load in flight.  Four iterations per round trip let the
+      // loads of the next three issue before the first is used (arithmetic stays in program order).  Measured on a
+      // 10 x 1e8 row sum: 2.6 -> 4.8 TB/s with 32 blocks per row, 320 -> 580 GB/s with one; 8 and 16 are no better.
+      bool plain = true;
+      visit_stmts(s->body, [&](const S& c) {
+        if (c->k == Stmt::Sync || c->k == Stmt::While || c->k == Stmt::RawStmt || (c->k == Stmt::For && !c->unroll)) plain = false;
+      });
+      if (plain) os << ind(n) << "#pragma unroll 4\n";
+    }
     os << ind(n) << "for (" << vty << " " << v << " = " << init(idx) << "; " << cond << "; " << v << " += "
        << (s->step * N) << ") {\n";
     pstmts(s->body, n + 2);

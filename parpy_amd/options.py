@@ -207,45 +207,66 @@ class CompileOptions:
     """src/option.rs:14-108; __str__ feeds the in-memory cache key (python/parpy/key.py:29-30)."""
 
     def __setattr__(self, name, value):
-        # every assignment to any options object gets a stamp that no other assignment has:
-        # (stamp, parallelize) identifies the state of an options object cheaply
+        # every assignment to any options object gets a stamp that no other assignment has;
+        # the stamp tells when the cached part of the fast key is stale
         _options_clock[0] += 1
         object.__setattr__(self, "_stamp", _options_clock[0])
         object.__setattr__(self, name, value)
 
     def _fast_key(self):
-        return (self._stamp, tuple((k, p.nthreads, p.reduction, p._tpb) for k, p in self.parallelize.items()))
+        """Hashable value of the whole options state: equal for two objects that hold equal settings,
+        so that a call with a freshly built options object finds the code compiled for an earlier one.
+        The fields assigned through attributes are cached per stamp; the containers, which can be
+        changed in place, are read every time."""
+        d = self.__dict__
+        if d.get("_key_stamp") != d["_stamp"]:
+            d["_key_fields"] = tuple(v for k, v in d.items()
+                                     if (k[0] != "_" or k in CompileOptions._DEFAULTS) and not isinstance(v, (dict, list)))
+            d["_key_stamp"] = d["_stamp"]
+        return (d["_key_fields"], tuple(d["includes"]), tuple(d["libs"]), tuple(d["extra_flags"]),
+                tuple((k, p.nthreads, p.reduction, p._tpb) for k, p in d["parallelize"].items()))
+
+    # opt_*: HIP memory-codegen switches; None keeps the compiler's default.  They exist so that
+    # tests and benchmarks can measure what each buys.
+    # defaults of the fields that hold plain values, in the order the fast key reads them
+    _DEFAULTS = {
+        'verbose_backend_resolution': False,
+        'debug_print': False,
+        'write_output': False,
+        'backend': CompileBackend.Auto,
+        'use_cuda_thread_block_clusters': False,
+        '_max_thread_blocks_per_cluster': 8,
+        'use_cuda_graphs': False,
+        '_force_int_size': None,
+        '_force_float_size': None,
+        'opt_vectorize': None,
+        'opt_lds_rows': None,
+        'opt_reg_cache': None,
+        'opt_hoist_invariant': None,
+        'opt_narrow_index': None,
+        'opt_mfma_sddmm': None,
+        'opt_unswitch': None,
+        'opt_gather_transpose': None,
+        'opt_nontemporal': None,
+        'opt_lane_split': None,
+        'opt_drop_barriers': None,
+        'opt_noalias_scopes': None,
+        'reg_budget': None,   # registers per thread the caching passes may claim (None: by block size)
+        'assume_aligned': None,   # set by the driver: False when an array argument is not 16-byte aligned
+    }
 
     def __init__(self):
-        self.parallelize = {}
-        self.verbose_backend_resolution = False
-        self.debug_print = False
-        self.write_output = False
-        self.backend = CompileBackend.Auto
-        self.use_cuda_thread_block_clusters = False
-        self._max_thread_blocks_per_cluster = 8
-        self.use_cuda_graphs = False
-        self._force_int_size = None
-        self._force_float_size = None
-        self.includes = []
-        self.libs = []
-        self.extra_flags = []
-        # HIP memory-codegen switches; None keeps the compiler's default (on).
-        # They exist so that tests and benchmarks can measure what each buys.
-        self.opt_vectorize = None
-        self.opt_lds_rows = None
-        self.opt_reg_cache = None
-        self.opt_hoist_invariant = None
-        self.opt_narrow_index = None
-        self.opt_mfma_sddmm = None
-        self.opt_unswitch = None
-        self.opt_gather_transpose = None
-        self.opt_nontemporal = None
-        self.opt_lane_split = None
-        self.opt_drop_barriers = None
-        self.opt_noalias_scopes = None
-        self.reg_budget = None       # registers per thread the caching passes may claim (None: by block size)
-        self.assume_aligned = None   # set by the driver: False when an array argument is not 16-byte aligned
+        # written into the instance dictionary directly: building an options object is part of
+        # many calls (`opts=parpy.par(...)`) and thirty stamped assignments would dominate them
+        d = self.__dict__
+        d.update(CompileOptions._DEFAULTS)
+        d["parallelize"] = {}
+        d["includes"] = []
+        d["libs"] = []
+        d["extra_flags"] = []
+        _options_clock[0] += 1
+        d["_stamp"] = d["_key_stamp"] = _options_clock[0]
+        d["_key_fields"] = CompileOptions._DEFAULT_KEY
 
     @property
     def max_thread_blocks_per_cluster(self):
@@ -291,6 +312,9 @@ class CompileOptions:
                 f"includes: {self.includes}, libs: {self.libs}, extra_flags: {self.extra_flags} }}")
 
 
+CompileOptions._DEFAULT_KEY = tuple(CompileOptions._DEFAULTS.values())
+
+
 class ScalarSizes:
     """Default scalar widths: int64 / float64 unless forced (src/utils/ast.rs:78-110)."""
 
@@ -305,5 +329,5 @@ def par(p):
     for k, v in p.items():
         if not isinstance(k, str) or not isinstance(v, LoopPar):
             raise TypeError("parallelization specification must map label strings to LoopPar values")
-    opts.parallelize = dict(p)
+    opts.__dict__["parallelize"] = dict(p)   # (no stamp needed: the fast key reads the mapping itself)
     return opts

@@ -127,6 +127,21 @@ def test_grid_wide_loop_is_vectorised_when_no_block_is_partial():
     assert not re.search(r"_u_\d+ < 4;", s.split("extern \"C\" __global__")[1])
 
 
+def test_rows_that_do_not_fill_the_block_are_still_vectorised_and_unrolled():
+    """A row of 10^7 floats over 1024 threads: whole vectors but a trip count that differs between threads.
+    The loop runs over vectors of four and asks for four iterations in flight; a row length that is no
+    multiple of four stays scalar (its rows are not 16-byte aligned)."""
+    x, y = np.zeros((2, 10**4), dtype=np.float32), np.zeros(2, dtype=np.float32)
+    s = compiles(parpy.print_compiled(W.sum_rows, [x, y, 2], opts_for({'outer': parpy.threads(2), 'inner': parpy.threads(1024)})))
+    body = s.split("extern \"C\" __global__")[1]
+    assert re.search(r"#pragma unroll 4\n\s+for \(int \w+_q_\d+ = \(int\)threadIdx.x; \w+ < 2500; \w+ \+= 1024\)", body)
+    assert re.search(r"_u_\d+ < 4;", body)
+    x = np.zeros((2, 10**4 + 2), dtype=np.float32)
+    s = compiles(parpy.print_compiled(W.sum_rows, [x, y, 2], opts_for({'outer': parpy.threads(2), 'inner': parpy.threads(1024)})))
+    body = s.split("extern \"C\" __global__")[1]
+    assert not re.search(r"_u_\d+ < 4;", body) and "< 10002;" in body
+
+
 def _hmm_args(k, n=4, maxlen=30):
     hmm, seqs = W.synthetic_hmm(k, n_inst=n, min_len=10, max_len=maxlen)
     S = hmm["num_states"]

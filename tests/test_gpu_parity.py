@@ -423,6 +423,27 @@ def test_repeated_calls_take_the_short_path_and_stay_correct():
         f(2.0, x, y, out, 1000, opts=o, extra=1)
 
 
+def test_a_fresh_options_object_with_equal_settings_takes_the_short_path():
+    """`opts=parpy.par(...)` builds a new options object per call (the reference's benchmarks and tests do):
+    equal settings must find the specialisation of the earlier call, different settings must not."""
+    f = parpy.jit(K.axpy)
+    x, y = torch.arange(512, dtype=torch.float32, device="cuda"), torch.ones(512, dtype=torch.float32, device="cuda")
+    out = torch.zeros(512, dtype=torch.float32, device="cuda")
+    for rep in range(5):
+        out.zero_()
+        f(2.0, x, y, out, 512, opts=parpy.par({'N': parpy.threads(128)}))      # backend Auto, resolved per call
+        assert torch.equal(out, 2.0 * x + y)
+    n_auto = len(f._seen_calls)
+    assert 1 <= n_auto <= 2
+    for rep in range(5):
+        f(2.0, x, y, out, 512, opts=opts_for({'N': parpy.threads(128)}))       # backend named
+    assert len(f._seen_calls) == n_auto
+    f(2.0, x, y, out, 512, opts=opts_for({'N': parpy.threads(64)}))
+    f(2.0, x, y, out, 512, opts=opts_for({'N': parpy.threads(128)}, opt_vectorize=False))
+    assert len(f._seen_calls) == n_auto + 2
+    assert torch.equal(out, 2.0 * x + y)
+
+
 def test_random_shapes_and_thread_counts():
     """Row reductions, softmax and the element-wise copy over seeded random shapes and thread counts:
     extents that do and do not divide by the vector width, the wavefront and the block size."""
