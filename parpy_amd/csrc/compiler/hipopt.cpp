@@ -71,9 +71,7 @@ bool thread_mapped(const S& s) { return s->k == Stmt::For && s->map.k == GpuMap:
 
 // iterations every thread runs in a thread-mapped loop, when that is a compile-time constant
 int64_t per_thread_trips(const S& loop) {
-  int64_t e = const_extent(loop);
-  if (e <= 0 || loop->map.n <= 0 || e % loop->map.n != 0) return -1;
-  return e / loop->map.n;
+  return counted_trips(const_extent(loop), loop->map.n);
 }
 
 // the per-thread iteration counter of a mapped loop as the printer names it

@@ -502,9 +502,11 @@ struct DevicePrinter {
       os << ind(n) << "}\n";
       return;
     }
-    if (const_bounds && extent % N == 0 && guard.empty()) {
-      // every thread runs the same, compile-time known number of iterations
-      int64_t per = extent / N;
+    if (const_bounds && guard.empty() && counted_trips(extent, N) > 0) {
+      // every thread runs the same, compile-time known number of iterations (the last one guarded when N does
+      // not divide the extent)
+      int64_t per = counted_trips(extent, N);
+      bool ragged = extent % N != 0;
       std::string k = v + "_k";
       {
         // the iteration counter can be named by the memory passes (register array slots)
@@ -518,7 +520,13 @@ struct DevicePrinter {
       if (s->unroll) os << ind(n) << "#pragma unroll\n";
       os << ind(n) << "for (int " << k << " = 0; " << k << " < " << per << "; ++" << k << ") {\n";
       os << ind(n + 2) << vty << " " << v << " = " << init("(" + idx + " + " + k + " * " + std::to_string(N) + ")") << ";\n";
-      pstmts(s->body, n + 2);
+      if (ragged) {
+        os << ind(n + 2) << "if (" << v << cmp << his << ") {\n";
+        pstmts(s->body, n + 4);
+        os << ind(n + 2) << "}\n";
+      } else {
+        pstmts(s->body, n + 2);
+      }
       os << ind(n) << "}\n";
       return;
     }

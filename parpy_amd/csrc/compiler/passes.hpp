@@ -37,6 +37,19 @@ struct Interval { bool known = false; int64_t lo = 0, hi = 0; };
 using RangeEnv = std::map<Name, Interval>;
 Interval expr_range(const E& e, const RangeEnv& env);
 
+// Iterations per thread of a loop of `extent` iterations spread over `n` threads when the loop is printed in
+// counted form (`for (k = 0; k < trips; ++k) v = tid + k*n`), -1 when it is printed as a strided loop instead.
+// Counted form gives every thread the same compile-time trip count, which is what lets the memory passes keep
+// per-iteration values in register arrays.  An extent that n does not divide is counted too as long as the trip
+// count stays small (the last iteration is guarded by `v < hi`); long ragged loops stay strided, where the
+// compiler can keep several unguarded loads in flight.
+inline int64_t counted_trips(int64_t extent, int64_t n) {
+  if (extent <= 0 || n <= 0) return -1;
+  if (extent % n == 0) return extent / n;
+  int64_t t = (extent + n - 1) / n;
+  return t <= 32 ? t : -1;
+}
+
 // ---- call time pipeline
 // specialise on the arguments, expand slices, type-check (specialize.cpp)
 FunDef specialize(const ParsedFun& pf, const std::vector<ArgDesc>& args, const Options& opts, NameGen& gen);

@@ -127,19 +127,32 @@ def test_grid_wide_loop_is_vectorised_when_no_block_is_partial():
     assert not re.search(r"_u_\d+ < 4;", s.split("extern \"C\" __global__")[1])
 
 
-def test_rows_that_do_not_fill_the_block_are_still_vectorised_and_unrolled():
-    """A row of 10^7 floats over 1024 threads: whole vectors but a trip count that differs between threads.
-    The loop runs over vectors of four and asks for four iterations in flight; a row length that is no
-    multiple of four stays scalar (its rows are not 16-byte aligned)."""
-    x, y = np.zeros((2, 10**4), dtype=np.float32), np.zeros(2, dtype=np.float32)
-    s = compiles(parpy.print_compiled(W.sum_rows, [x, y, 2], opts_for({'outer': parpy.threads(2), 'inner': parpy.threads(1024)})))
-    body = s.split("extern \"C\" __global__")[1]
-    assert re.search(r"#pragma unroll 4\n\s+for \(int \w+_q_\d+ = \(int\)threadIdx.x; \w+ < 2500; \w+ \+= 1024\)", body)
+def test_rows_that_do_not_fill_the_block_are_still_vectorised():
+    """Whole vectors but a trip count that differs between threads.  A long row (10^6 floats over 1024 threads)
+    is a strided loop over vectors of four that asks for four iterations in flight; a short one (10^4 floats,
+    three vectors per thread at most) is a counted loop whose iterations are guarded, which keeps the per-thread
+    register arrays of the caching passes; a row length that is no multiple of four stays scalar (its rows are
+    not 16-byte aligned)."""
+    par = opts_for({'outer': parpy.threads(2), 'inner': parpy.threads(1024)})
+    x, y = np.zeros((2, 10**6), dtype=np.float32), np.zeros(2, dtype=np.float32)
+    body = compiles(parpy.print_compiled(W.sum_rows, [x, y, 2], par)).split("extern \"C\" __global__")[1]
+    assert re.search(r"#pragma unroll 4\n\s+for \(int \w+_q_\d+ = \(int\)threadIdx.x; \w+ < 250000; \w+ \+= 1024\)", body)
     assert re.search(r"_u_\d+ < 4;", body)
+    x = np.zeros((2, 10**4), dtype=np.float32)
+    body = compiles(parpy.print_compiled(W.sum_rows, [x, y, 2], par)).split("extern \"C\" __global__")[1]
+    assert re.search(r"_k < 3;", body) and re.search(r"if \(\w+_q_\d+ < 2500\) \{", body) and re.search(r"_u_\d+ < 4;", body)
     x = np.zeros((2, 10**4 + 2), dtype=np.float32)
-    s = compiles(parpy.print_compiled(W.sum_rows, [x, y, 2], opts_for({'outer': parpy.threads(2), 'inner': parpy.threads(1024)})))
+    body = compiles(parpy.print_compiled(W.sum_rows, [x, y, 2], par)).split("extern \"C\" __global__")[1]
+    assert not re.search(r"_u_\d+ < 4;", body) and "< 10002" in body
+
+
+def test_softmax_rows_stay_in_registers_when_the_block_does_not_divide_them():
+    N, M = 64, 1000
+    x = np.zeros((N, M), dtype=np.float32)
+    s = compiles(parpy.print_compiled(W.softmax, [x, N, M, x.copy()], opts_for({'N': parpy.threads(N), 'M': parpy.threads(64)})))
     body = s.split("extern \"C\" __global__")[1]
-    assert not re.search(r"_u_\d+ < 4;", body) and "< 10002;" in body
+    assert len(re.findall(r"= x_\d+\[", body)) == 1 and len(re.findall(r"&out_\d+\[", body)) == 1
+    assert len(re.findall(r"if \(\w+ < 250\) \{", body)) == 4
 
 
 def _hmm_args(k, n=4, maxlen=30):
