@@ -13,6 +13,7 @@
 #include <cmath>
 #include <cstring>
 #include <map>
+#include <mutex>
 #include <string>
 #include <vector>
 
@@ -119,6 +120,10 @@ struct Plan {
   std::vector<void*> graph_args;
   int64_t graph_launches = 0;
   int64_t graph_replays = 0;           // runs served by hipGraphLaunch so far
+  // A run writes the plan's variable slots and temporaries, and callers reach this library through
+  // foreign-function calls that release the interpreter lock: two threads calling one compiled
+  // function must take turns (the device work they enqueue is ordered by the stream anyway).
+  std::mutex mu;
 };
 
 struct PlanBuilder {
@@ -631,14 +636,18 @@ extern "C" {
 
 int32_t parpy_hip_plan_set_graph(void* plan, int32_t enable) {
   Plan& p = *(Plan*)plan;
+  std::lock_guard<std::mutex> turn(p.mu);
   p.use_graph = enable != 0;
   if (!p.use_graph) drop_graph(p);
   p.graph_state = 0;
   return 0;
 }
 
-int32_t parpy_hip_plan_run(void* plan, void* const* args, int32_t nargs) {
-  Plan& p = *(Plan*)plan;
+}  // extern "C"
+
+namespace {
+
+int32_t plan_run_locked(Plan& p, void* const* args, int32_t nargs) {
   if (nargs != p.nparams)
     return fail("launch plan expects " + std::to_string(p.nparams) + " pointer arguments, received " + std::to_string(nargs));
   if (!p.module) return fail("launch plan was created without a loaded module");
@@ -662,14 +671,25 @@ int32_t parpy_hip_plan_run(void* plan, void* const* args, int32_t nargs) {
   return rc;
 }
 
+}  // namespace
+
+extern "C" {
+
+int32_t parpy_hip_plan_run(void* plan, void* const* args, int32_t nargs) {
+  Plan& p = *(Plan*)plan;
+  std::lock_guard<std::mutex> turn(p.mu);
+  return plan_run_locked(p, args, nargs);
+}
+
 int32_t parpy_hip_plan_run_timed(void* plan, void* const* args, int32_t nargs, float* elapsed_ms) {
   Plan& p = *(Plan*)plan;
+  std::lock_guard<std::mutex> turn(p.mu);
   if (!p.ev_start) {
     if (int32_t rc = check(hipEventCreate(&p.ev_start), "hipEventCreate")) return rc;
     if (int32_t rc = check(hipEventCreate(&p.ev_stop), "hipEventCreate")) return rc;
   }
   if (int32_t rc = check(hipEventRecord(p.ev_start, nullptr), "hipEventRecord")) return rc;
-  if (int32_t rc = parpy_hip_plan_run(plan, args, nargs)) return rc;
+  if (int32_t rc = plan_run_locked(p, args, nargs)) return rc;
   if (int32_t rc = check(hipEventRecord(p.ev_stop, nullptr), "hipEventRecord")) return rc;
   if (int32_t rc = check(hipEventSynchronize(p.ev_stop), "hipEventSynchronize")) return rc;
   return check(hipEventElapsedTime(elapsed_ms, p.ev_start, p.ev_stop), "hipEventElapsedTime");

@@ -444,6 +444,36 @@ def test_a_fresh_options_object_with_equal_settings_takes_the_short_path():
     assert torch.equal(out, 2.0 * x + y)
 
 
+def test_two_host_threads_share_one_compiled_function():
+    """Foreign-function calls release the interpreter lock, so two Python threads can be inside the runtime at
+    once; runs of one launch plan (host loop state, kept temporaries) must take turns."""
+    import threading
+    N, M = 8, 8192
+    f = parpy.jit(K.sum_rows)
+    o = opts_for({'outer': parpy.threads(N), 'inner': parpy.threads(2048)})    # two blocks per row: a temporary and two kernels
+    xs = [torch.randn((N, M), dtype=torch.float64, device="cuda") for _ in range(2)]
+    outs = [torch.zeros(N, dtype=torch.float64, device="cuda") for _ in range(2)]
+    f(xs[0], outs[0], N, opts=o)
+    bad = []
+
+    def work(i):
+        for rep in range(200):
+            outs[i].zero_()
+            f(xs[i], outs[i], N, opts=o)
+            if rep % 50 == 49 and not torch.allclose(outs[i], xs[i].sum(dim=1), rtol=1e-12, atol=1e-12):
+                bad.append((i, rep))
+
+    ts = [threading.Thread(target=work, args=(i,)) for i in range(2)]
+    for t in ts:
+        t.start()
+    for t in ts:
+        t.join()
+    torch.cuda.synchronize()
+    assert not bad
+    for i in range(2):
+        assert torch.allclose(outs[i], xs[i].sum(dim=1), rtol=1e-12, atol=1e-12)
+
+
 def test_random_shapes_and_thread_counts():
     """Row reductions, softmax and the element-wise copy over seeded random shapes and thread counts:
     extents that do and do not divide by the vector width, the wavefront and the block size."""
