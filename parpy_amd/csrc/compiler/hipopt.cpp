@@ -1377,12 +1377,12 @@ struct GatherTranspose {
     px.read_only = true;
     pxt.id = xt;
     pxt.ty = Type::pointer(c.sz);
-    if (c.K % 64 == 0 && c.N % 64 == 0 && elem_bytes(c.sz) >= 4) {
-      // whole 64 x 64 tiles: turned round in LDS by a device helper, whole lines on both sides
+    if (c.K >= 16 && c.N >= 64 && elem_bytes(c.sz) >= 4) {
+      // 64 x 64 tiles turned round in LDS by a device helper, whole lines on both sides (edge tiles are guarded)
       Kernel k;
       k.name = p.name + "_transpose_" + x.s + "_" + std::to_string(gen.next++);
-      k.grid.x = c.N / 64;
-      k.grid.y = c.K / 64;
+      k.grid.x = (c.N + 63) / 64;
+      k.grid.y = (c.K + 63) / 64;
       k.block.x = 256;
       k.lds_bytes = 64 * 65 * elem_bytes(c.sz);
       k.cached_stores = true;
@@ -1558,7 +1558,7 @@ struct LaneSplit {
       v = v == 0 ? w : std::min(v, w);
       ++loads;
     });
-    if (!ok || loads < 1 || s->hi->iv % (v * G) != 0 || s->hi->iv < 4 * v * G) return false;
+    if (!ok || loads < 1 || s->hi->iv % v != 0 || s->hi->iv < 2 * v * G) return false;  // whole vectors, and enough of them
     *vec = v;
     *term_out = term;
     return true;
@@ -1638,8 +1638,16 @@ struct LaneSplit {
     inner->unroll = true;
     auto outer = clone(loop);
     outer->id = d0;
-    outer->hi = mk_int(loop->hi->iv / (vec * G), isz);
-    outer->body = {S(inner)};
+    const int64_t K = loop->hi->iv, chunk = vec * G;
+    outer->hi = mk_int((K + chunk - 1) / chunk, isz);
+    if (K % chunk == 0) {
+      outer->body = {S(inner)};
+    } else {
+      // the last round covers only part of the group: lanes whose vector starts past the end sit it out
+      E base = mk_binop(BinOp::Mul, mk_binop(BinOp::Add, mk_binop(BinOp::Mul, mk_var(d0, ity), mk_int(G, isz), ity), gv, ity),
+                        mk_int(vec, isz), ity);
+      outer->body = {mk_if(mk_binop(BinOp::Lt, base, mk_int(K, isz), Type::scalar(ElemSize::Bool)), {S(inner)}, {})};
+    }
     body.push_back(outer);
     body.push_back(mk_assign(t, mk_raw("parpy_sum8(" + t->name.str() + ")", t->ty)));
     Stmts stores;

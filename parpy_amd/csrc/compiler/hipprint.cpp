@@ -163,16 +163,23 @@ typedef float parpy_f32x4 __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ int parpy_lane_id() { return (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)); }
 // dst[c][r] = src[r][c] for a ROWS x COLS matrix in 64 x 64 tiles: a 256-thread workgroup reads
 // 64-word row segments of its tile, turns the tile round in LDS and writes 64-word row segments
-// of the result, so both sides move whole 256-byte lines.  Launched on a (COLS/64, ROWS/64) grid.
+// of the result, so both sides move whole 256-byte lines.  Launched on a (ceil(COLS/64), ceil(ROWS/64))
+// grid; the bounds tests of the edge tiles are compile-time false when 64 divides the extents.
 template <class T, int ROWS, int COLS> __device__ __forceinline__ void parpy_transpose_tile(const T* __restrict__ src, T* __restrict__ dst) {
   __shared__ T tile[64][65];
   const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
   const int c0 = (int)blockIdx.x * 64, r0 = (int)blockIdx.y * 64;
   #pragma unroll
-  for (int j = 0; j < 16; ++j) tile[j * 4 + ty][tx] = src[(long long)(r0 + j * 4 + ty) * COLS + c0 + tx];
+  for (int j = 0; j < 16; ++j) {
+    const int r = r0 + j * 4 + ty, c = c0 + tx;
+    if ((ROWS % 64 == 0 || r < ROWS) && (COLS % 64 == 0 || c < COLS)) tile[j * 4 + ty][tx] = src[(long long)r * COLS + c];
+  }
   __syncthreads();
   #pragma unroll
-  for (int j = 0; j < 16; ++j) dst[(long long)(c0 + j * 4 + ty) * ROWS + r0 + tx] = tile[tx][j * 4 + ty];
+  for (int j = 0; j < 16; ++j) {
+    const int c = c0 + j * 4 + ty, r = r0 + tx;
+    if ((COLS % 64 == 0 || c < COLS) && (ROWS % 64 == 0 || r < ROWS)) dst[(long long)c * ROWS + r] = tile[tx][j * 4 + ty];
+  }
 }
 )";
 

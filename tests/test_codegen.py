@@ -219,8 +219,14 @@ def test_sddmm_kernels_compile():
     C = {"rows": rows, "cols": cols, "values": vals, "nnz": len(cols)}
     s = compiles(parpy.print_compiled(W.sddmm_coo, [A, B, C, np.zeros_like(vals), 1.5, 2.0], opts_for({"nnz": parpy.threads(len(cols))})))
     # the column gather B[:, col] is staged through a transposed temporary first
-    assert launch(s) == [("1", "1", "1", "128", "1", "1"), ("1", "1", "1", "832", "1", "1")]
-    assert "B_T_" in s and "parpy_alloc_buffer(8192)" in s
+    # (16 x 128: two 64 x 64 tiles whose lower 48 rows are guarded away)
+    assert launch(s) == [("2", "1", "1", "256", "1", "1"), ("1", "1", "1", "832", "1", "1")]
+    assert "B_T_" in s and "parpy_alloc_buffer(8192)" in s and "parpy_transpose_tile<float, 16, 128>(" in s
+    # a matrix too thin for tiles is transposed by one thread per column
+    A1, B1, crows1, cols1, vals1 = W.make_sddmm(128, 8, 0.05)
+    C1 = {"rows": oracle.csr_rows(crows1), "cols": cols1, "values": vals1, "nnz": len(cols1)}
+    s1 = compiles(parpy.print_compiled(W.sddmm_coo, [A1, B1, C1, np.zeros_like(vals1), 1.5, 2.0], opts_for({"nnz": parpy.threads(len(cols1))})))
+    assert launch(s1)[0] == ("1", "1", "1", "128", "1", "1") and "parpy_transpose_tile" not in s1.split("extern \"C\" __global__", 1)[1]
     s0 = compiles(parpy.print_compiled(W.sddmm_coo, [A, B, C, np.zeros_like(vals), 1.5, 2.0],
                                        opts_for({"nnz": parpy.threads(len(cols))}, opt_gather_transpose=False)))
     assert launch(s0) == [("1", "1", "1", "832", "1", "1")]
@@ -243,6 +249,12 @@ def test_sddmm_kernels_compile():
     sn = compiles(parpy.print_compiled(W.sddmm_coo, [A3, B3, C3, np.zeros_like(vals3), 1.5, 2.0],
                                        opts_for({"nnz": parpy.threads(n3).tpb(256)}, opt_lane_split=False)))
     assert "parpy_sum8(t_" not in sn and launch(sn)[1][0] == str((n3 + 255) // 256)
+    # an inner extent the lane group does not divide (100 = 3 rounds of 32 + 4): the lanes past the end skip the last round
+    A4, B4, crows4, cols4, vals4 = W.make_sddmm(1000, 100, 0.01)
+    C4 = {"rows": oracle.csr_rows(crows4), "cols": cols4, "values": vals4, "nnz": len(cols4)}
+    sr = compiles(parpy.print_compiled(W.sddmm_coo, [A4, B4, C4, np.zeros_like(vals4), 1.5, 2.0], opts_for({"nnz": parpy.threads(len(cols4)).tpb(256)})))
+    assert "parpy_sum8(t_" in sr and re.search(r"_c_\d+ < 4;", sr) and re.search(r"\* 4\) < 100\) \{", sr)
+    assert "parpy_transpose_tile<float, 100, 1000>(" in sr and launch(sr)[0] == ("16", "2", "1", "256", "1", "1")
     s = compiles(parpy.print_compiled(W.sddmm_decompress_csr, [crows, np.zeros_like(cols), 128],
                                       opts_for({"N": parpy.threads(128), "M": parpy.threads(64)})))
     assert launch(s) == [("1", "128", "1", "64", "1", "1")]

@@ -510,7 +510,8 @@ def test_random_sddmm_and_hmm_configurations():
     multiples of 32 and 64 (lane groups, tiled transposition), few and many non-zeros, state counts
     below and above one workgroup, odd thread counts."""
     rng = np.random.default_rng(77)
-    for n, k, density in [(64, 8, 0.2), (100, 48, 0.1), (512, 96, 0.05), (640, 128, 0.02), (1000, 200, 0.01), (2048, 64, 0.01)]:
+    for n, k, density in [(64, 8, 0.2), (100, 48, 0.1), (512, 96, 0.05), (640, 128, 0.02), (1000, 200, 0.01), (2048, 64, 0.01),
+                          (777, 100, 0.02), (300, 36, 0.1), (1500, 68, 0.01)]:
         A, B, crows, cols, vals = W.make_sddmm(n, k, density, seed=int(rng.integers(1 << 30)))
         rows = oracle.csr_rows(crows)
         nnz = len(cols)
