@@ -942,32 +942,52 @@ struct Pass {
     };
     scan_stmts(k.body, -1, false);
 
-    struct Chosen { Name arr, reg; ElemSize sz; E inv; int first, last_write; bool load_first; };
+    struct Chosen { Name arr, reg; ElemSize sz; E inv; int first, last, last_write; bool load_first; int64_t cost; };
     std::vector<Chosen> chosen;
     int64_t slots = group[0].is.slots;
+    // Registers are budgeted by what is live at once, loop by loop: an array occupies its slots from the first
+    // loop that touches it to the last.  Where one array is read for the last time in the very loop that first
+    // writes another (out[e] = f(x[e]) with x dead afterwards), each iteration frees a slot as it fills one,
+    // so the pair needs the larger of the two, not the sum.
+    const int G = (int)group.size();
+    auto peak_with = [&](const std::vector<Chosen>& cs) {
+      int64_t peak = 0;
+      for (int g = 0; g < G; ++g) {
+        int64_t live = 0, dying = 0, born = 0;
+        for (auto& c : cs) {
+          if (c.first > g || c.last < g) continue;
+          live += c.cost;
+          if (c.last == g && c.first < g) dying += c.cost;
+          if (c.first == g && !c.load_first && c.last > g) born += c.cost;
+        }
+        peak = std::max(peak, live - std::min(dying, born));
+      }
+      return peak;
+    };
     for (auto& p : k.params) {
       auto it = arrs.find(p.id);
       if (it == arrs.end() || !it->second.ok || !it->second.seen) continue;
       const Arr& a = it->second;
-      int touched = 0, first = -1, last_write = -1;
+      int touched = 0, first = -1, last = -1, last_write = -1;
       for (size_t g = 0; g < group.size(); ++g) {
-        if (a.reads[g] || a.writes[g]) { ++touched; if (first < 0) first = (int)g; }
+        if (a.reads[g] || a.writes[g]) { ++touched; if (first < 0) first = (int)g; last = (int)g; }
         if (a.writes[g]) last_write = (int)g;
       }
       if (touched < 2) continue;
-      int64_t cost = slots * std::max(1, elem_bytes(a.sz) / 4);
-      if (*budget < cost) continue;
-      *budget -= cost;
       Chosen c;
       c.arr = p.id;
-      c.reg = gen.fresh("row_" + p.id.s);
       c.sz = a.sz;
       c.inv = a.inv;
       c.first = first;
+      c.last = last;
       c.last_write = last_write;
       c.load_first = a.reads[first];
+      c.cost = slots * std::max(1, elem_bytes(a.sz) / 4);
       chosen.push_back(c);
+      if (peak_with(chosen) > *budget) { chosen.pop_back(); continue; }
+      chosen.back().reg = gen.fresh("row_" + p.id.s);
     }
+    if (!chosen.empty()) *budget -= peak_with(chosen);
     if (chosen.empty()) return;
 
     Type ity = Type::scalar(isz);

@@ -117,6 +117,21 @@ def test_softmax_is_one_kernel_and_row_resident():
     assert len(re.findall(r"x_\d+\[", s0.split("extern \"C\" __global__")[1])) >= 2
 
 
+def test_register_budget_counts_what_is_live_at_once():
+    """A 65536-float row on 1024 threads is 64 values per thread; x dies in the loop that first writes out, so the
+    two arrays take turns in the same registers and both are cached (1 read + 1 write per element)."""
+    N, M = 4, 65536
+    x = np.zeros((N, M), dtype=np.float32)
+    s = compiles(parpy.print_compiled(W.softmax, [x, N, M, x.copy()], opts_for({'N': parpy.threads(N), 'M': parpy.threads(1024)})))
+    body = s.split("extern \"C\" __global__")[1]
+    assert len(re.findall(r"= x_\d+\[", body)) == 1 and len(re.findall(r"&out_\d+\[", body)) == 1
+    assert "float row_x_" in body and "float row_out_" in body
+    # twice the row: nothing fits any more and the four statements go through memory
+    x = np.zeros((N, 2 * M), dtype=np.float32)
+    s = compiles(parpy.print_compiled(W.softmax, [x, N, 2 * M, x.copy()], opts_for({'N': parpy.threads(N), 'M': parpy.threads(1024)})))
+    assert "float row_" not in s.split("extern \"C\" __global__")[1]
+
+
 def test_grid_wide_loop_is_vectorised_when_no_block_is_partial():
     n = 1 << 20
     x = np.zeros(n, dtype=np.float32)
