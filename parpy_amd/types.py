@@ -1,21 +1,13 @@
-"""Short aliases for element sizes (python/parpy/types.py:1-20)."""
+"""Short names for element types: `parpy.types.F32` is `ElemSize.F32`, and so on for every member
+(python/parpy/types.py:1-20 of the reference), plus the pointer type of an external's parameter."""
 from .options import ElemSize, ExtType
 
-Bool = ElemSize.Bool
-I8 = ElemSize.I8
-I16 = ElemSize.I16
-I32 = ElemSize.I32
-I64 = ElemSize.I64
-U8 = ElemSize.U8
-U16 = ElemSize.U16
-U32 = ElemSize.U32
-U64 = ElemSize.U64
-F16 = ElemSize.F16
-F32 = ElemSize.F32
-F64 = ElemSize.F64
+globals().update({member.name: member for member in ElemSize})
+__all__ = [member.name for member in ElemSize] + ["pointer"]
 
 
 def pointer(ty):
-    if isinstance(ty, ElemSize):
-        return ExtType.Pointer(ty)
-    raise RuntimeError(f"Provided type {ty} must be an ExtType.")
+    """Type of a pointer parameter of an external function whose elements have type `ty`."""
+    if not isinstance(ty, ElemSize):
+        raise RuntimeError(f"Provided type {ty} must be an ExtType.")
+    return ExtType.Pointer(ty)
