@@ -24,33 +24,23 @@ _ext_tops = {}
 _fun_cache = {}
 
 
-def _get_tops(backend):
-    ast_tops = {k.__name__: v for k, v in _ir_asts.items()}
-    if backend is not None:
-        ext_tops = _ext_decls.get(backend, {})
-    else:
-        ext_tops = _ext_tops
-    return {**ast_tops, **ext_tops}
-
-
-def _get_source_code(fn):
-    import inspect
-    import itertools
-    import textwrap
-    src, fst_line = inspect.getsourcelines(fn)
-    col_ofs = sum(1 for _ in itertools.takewhile(str.isspace, src[0]))
-    src = textwrap.dedent("".join(src))
-    return src, fst_line - 1, col_ofs
+def _callable_names(backend):
+    """What a call inside a jitted function may refer to: every function jitted so far, and the externals
+    declared for `backend` (all externals, by name only, while a function is being parsed)."""
+    names = {f.__name__: ir for f, ir in _ir_asts.items()}
+    names.update(_ext_tops if backend is None else _ext_decls.get(backend, {}))
+    return names
 
 
 def _convert_python_function_to_ir(fn, vars):
     import ast as python_ast
     import inspect
-    filepath = inspect.getfile(fn)
-    src, line_ofs, col_ofs = _get_source_code(fn)
-    tree = python_ast.parse(src)
-    top_map = _get_tops(None)
-    info = (filepath, line_ofs, col_ofs)
+    import textwrap
+    lines, first_line = inspect.getsourcelines(fn)
+    indent = len(lines[0]) - len(lines[0].lstrip())
+    tree = python_ast.parse(textwrap.dedent("".join(lines)))
+    # positions in error messages refer to the file, not to the dedented excerpt
+    info = (inspect.getfile(fn), first_line - 1, indent)
     # Names are resolved the way Python itself would for `fn` -- closure cells,
     # then the globals of the module that defines it -- with the caller's frame
     # (what the reference consults, python/parpy/__init__.py:235-237) as fallback.
@@ -61,22 +51,17 @@ def _convert_python_function_to_ir(fn, vars):
     except (TypeError, ValueError):
         nonlocals = {}
     locs = {**caller_locs, **nonlocals} if caller_locs is not caller_globs else nonlocals
-    return compiler.python_to_ir(tree, info, top_map, (globs, locs))
+    return compiler.python_to_ir(tree, info, _callable_names(None), (globs, locs))
 
 
-def _check_kwarg(kwargs, key, expected_ty, fun_name):
-    if key not in kwargs or kwargs[key] is None:
-        raise RuntimeError(f"Missing required keyword argument {key} in call to {fun_name}")
-    if isinstance(kwargs[key], expected_ty):
-        v = kwargs[key]
-        del kwargs[key]
-        return v
-    raise RuntimeError(f"The keyword argument {key} should be of type {expected_ty}")
-
-
-def _check_kwargs(kwargs, fun_name):
-    opts = _check_kwarg(kwargs, "opts", CompileOptions, fun_name)
-    if len(kwargs) > 0:
+def _take_opts(kwargs, fun_name):
+    """The `opts` keyword of a call to a jitted function; it is required and nothing else is accepted."""
+    opts = kwargs.pop("opts", None)
+    if opts is None:
+        raise RuntimeError(f"Missing required keyword argument opts in call to {fun_name}")
+    if not isinstance(opts, CompileOptions):
+        raise RuntimeError(f"The keyword argument opts should be of type {CompileOptions}")
+    if kwargs:
         raise RuntimeError(f"Received unsupported keyword arguments: {kwargs}")
     return opts
 
@@ -103,7 +88,7 @@ def _compile_function(ir_ast, args, opts):
     fast_cache_key = _generate_fast_cache_key(ir_ast, args, opts)
     if fast_cache_key in _fun_cache:
         return _fun_cache[fast_cache_key]
-    top_map = _get_tops(opts.backend)
+    top_map = _callable_names(opts.backend)
     res = compiler.compile_ir(ir_ast, args, opts, top_map)
     cache_key = _generate_function_key(res.device_src, opts)
     build_code_object(cache_key, res.device_src, opts)
@@ -168,7 +153,7 @@ def print_compiled(fun, args, opts=None):
         locs = inspect.currentframe().f_back.f_locals
         ir_ast = _convert_python_function_to_ir(fun, (globs, locs))
     args = check_arguments(args, opts, False)
-    top_map = _get_tops(opts.backend)
+    top_map = _callable_names(opts.backend)
     return compiler.compile_ir(ir_ast, args, opts, top_map).listing
 
 
@@ -279,7 +264,7 @@ def jit(fun):
                     return hit.run_pointers(call[1])
         else:
             call = key = None
-        opts = backend._resolve_backend(_check_kwargs(kwargs, fun.__name__), True)
+        opts = backend._resolve_backend(_take_opts(kwargs, fun.__name__), True)
         checked = check_arguments(args, opts, True)
         wrap_fn = _compile_function(ir_ast, checked, opts)
         wrap_fn(*checked)
