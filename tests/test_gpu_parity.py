@@ -161,6 +161,36 @@ def test_forward_5mer_golden(golden_dir):
     assert np.allclose(got, exp, atol=1e-5, rtol=1e-5), np.abs(got - exp).max()
 
 
+def _random_reference_model(k, n_reads, max_len, seed):
+    """Tables in the reference model's format (16 duration layers over 4^k k-mers) with random contents."""
+    rng = np.random.default_rng(seed)
+    nk = 4 ** k
+    tail = 0.05
+    hmm = {
+        "trans1": np.log(rng.dirichlet(np.ones(4), size=nk)).astype(np.float32),          # [4^k, 4]
+        "trans2": np.log(rng.dirichlet(np.ones(16))).astype(np.float32),
+        "output_prob": np.ascontiguousarray(np.log(rng.dirichlet(np.ones(101), size=nk)).T.astype(np.float32)),
+        "initial_prob": np.concatenate([np.full(nk, -np.log(float(nk))), np.full(15 * nk, -np.inf)]).astype(np.float32),
+        "gamma": np.float32(np.log(tail)),
+        "synthetic_248": np.float32(np.log1p(-tail)),
+        "num_states": 16 * nk,
+    }
+    lens = rng.integers(2, max_len + 1, size=n_reads).astype(np.int64)
+    data = rng.integers(0, 101, size=(n_reads, int(lens.max()))).astype(np.int8)
+    seqs = {"data": data, "lens": lens, "maxlen": int(lens.max()), "num_instances": n_reads}
+    return hmm, seqs
+
+
+@pytest.mark.parametrize("threads", [1024, 16384])
+def test_reference_model_with_state_vectors_larger_than_lds(threads):
+    """A 6-mer model in the reference's format has 65536 states: one state vector is 256 KiB and stays in global
+    memory, in one workgroup per read and with the time loop on the host over 16 workgroups per read."""
+    hmm, seqs = _random_reference_model(6, n_reads=3, max_len=12, seed=11)
+    got = _run_reference_model(hmm, seqs, threads)
+    want = oracle.hmm_ref_forward(hmm, seqs, np.float32)
+    assert np.all(np.isfinite(want)) and np.allclose(got, want, atol=1e-4, rtol=1e-5), np.abs(got - want).max()
+
+
 def _run_synthetic(hmm, seqs, threads, **kw):
     hd, sd = W.to_device(hmm), W.to_device(seqs)
     n, S = seqs["num_instances"], hmm["num_states"]
