@@ -550,7 +550,8 @@ def test_random_sddmm_and_hmm_configurations():
         W.sddmm_coo(torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda(), C, D, 0.5, -1.5, opts=opts_for({"nnz": parpy.threads(nnz).tpb(256)}))
         want = oracle.sddmm(A, B, rows, cols, vals, alpha=0.5, beta=-1.5)
         assert np.allclose(D.cpu().numpy(), want, atol=1e-4, rtol=1e-5), (n, k, density)
-    for k, threads, n_inst, max_len in [(2, 64, 3, 40), (3, 100, 5, 77), (4, 128, 7, 33), (5, 512, 4, 150), (6, 1024, 3, 60), (6, 2048, 2, 25)]:
+    for k, threads, n_inst, max_len in [(2, 64, 3, 40), (3, 100, 5, 77), (4, 128, 7, 33), (5, 512, 4, 150), (6, 1024, 3, 60), (6, 2048, 2, 25),
+                                       (5, 192, 3, 50), (4, 96, 2, 31), (6, 640, 2, 20), (6, 3072, 2, 20)]:
         hmm, seqs = W.synthetic_hmm(k, n_inst=n_inst, min_len=2, max_len=max_len, seed=int(rng.integers(1 << 30)))
         got, _, _ = _run_synthetic(hmm, seqs, threads)
         want = oracle.hmm_syn_forward(hmm, seqs, np.float32)
