@@ -1598,11 +1598,15 @@ struct LaneSplit {
   bool apply(Kernel& k, const StmtP& launch) {
     if (k.body.size() != 1) return false;
     const S& root = k.body[0];
-    if (!(root->k == Stmt::For && root->map.k == GpuMap::ThreadBlock && root->map.dim == 0 && root->step == 1 &&
+    // the iterations of the whole launch: spread over the grid, or over the threads of a single workgroup
+    // (which then becomes a grid, since eight times as many threads may not fit one workgroup)
+    bool one_group = root->k == Stmt::For && root->map.k == GpuMap::Thread && k.grid.x == 1;
+    if (!(root->k == Stmt::For && (root->map.k == GpuMap::ThreadBlock || one_group) && root->map.dim == 0 && root->step == 1 &&
           root->lo->k == Expr::Int && root->lo->iv == 0 && root->hi->k == Expr::Int))
       return false;
     int64_t N = root->hi->iv;
-    if (N < 4096 || k.grid.y != 1 || k.grid.z != 1 || k.block.y != 1 || k.block.z != 1) return false;  // small launches gain nothing
+    if (one_group && N > root->map.n) return false;  // a strided loop inside the workgroup: iterations are not one per thread
+    if (N < 64 || k.grid.y != 1 || k.grid.z != 1 || k.block.y != 1 || k.block.z != 1) return false;  // (less than a wavefront of iterations: nothing to share)
     int pos = -1, vec = 0;
     E term;
     for (size_t q = 0; q < root->body.size(); ++q) {
@@ -1700,11 +1704,15 @@ struct LaneSplit {
     nr->id = gi;
     nr->hi = mk_int(N * G, isz);
     nr->body = body;
-    int64_t tpb = root->map.tpb;
+    int64_t tpb = one_group ? 256 : root->map.tpb;
+    nr->map.k = GpuMap::ThreadBlock;
+    nr->map.tpb = tpb;
     nr->map.n = (N * G + WAVE_SIZE - 1) / WAVE_SIZE * WAVE_SIZE;
     k.body = {S(nr)};
+    k.block.x = tpb;
     k.grid.x = (nr->map.n + tpb - 1) / tpb;
     launch->grid = k.grid;
+    launch->block = k.block;
     return true;
   }
 

@@ -79,6 +79,17 @@ def test_one_thread_per_row_on_many_rows(lane_split):
     assert np.allclose(out, x.astype(np.float64).sum(axis=1), atol=1e-4, rtol=1e-5)
 
 
+@pytest.mark.parametrize("rows,cols", [(100, 2048), (1024, 516), (64, 64), (1000, 100)])
+def test_one_thread_per_row_inside_one_workgroup(rows, cols):
+    """Few rows, one thread each, all in one workgroup: the lane groups turn the launch into a grid of their own;
+    row counts that do not fill the last workgroup and row lengths that the group of eight does not divide."""
+    x = np.random.default_rng(rows).uniform(-1, 1, (rows, cols)).astype(np.float32)
+    for split in (True, False):
+        out = np.zeros(rows, dtype=np.float32)
+        parpy.jit(K.sum_rows)(x, out, rows, opts=opts_for({'outer': parpy.threads(rows)}, opt_lane_split=split))
+        assert np.allclose(out, x.astype(np.float64).sum(axis=1), atol=1e-4, rtol=1e-5), (rows, cols, split)
+
+
 @pytest.mark.parametrize("threads", [64, 2048])
 def test_strided_reduction(threads):
     N, M = 10, 4096
