@@ -68,6 +68,19 @@ def sddmm_coo(A, B, C, D, alpha, beta):
         D[i] = alpha * t + beta * C["values"][i]
 
 
+@parpy.jit
+def sddmm_csr(A, B, C, D, N, alpha, beta):
+    """SDDMM on a CSR mask: the row pointers are decompressed into `C["rows"]` by a call to the kernel
+    above, then the non-zeros are processed as in the COO form (benchmarks/sddmm.py:29-42)."""
+    sddmm_decompress_csr(C["crows"], C["rows"], N)
+    parpy.label('nnz')
+    for i in range(C["nnz"]):
+        row = C["rows"][i]
+        col = C["cols"][i]
+        t = sum(A[row, :] * B[:, col])
+        D[i] = alpha * t + beta * C["values"][i]
+
+
 # ---------------------------------------------------------------- HMM forward, reference (16-layer) model
 @parpy.jit
 def forward_kernel(hmm, seqs, alpha1, alpha2, result):

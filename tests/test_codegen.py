@@ -270,6 +270,13 @@ def test_sddmm_kernels_compile():
     sr = compiles(parpy.print_compiled(W.sddmm_coo, [A4, B4, C4, np.zeros_like(vals4), 1.5, 2.0], opts_for({"nnz": parpy.threads(len(cols4)).tpb(256)})))
     assert "parpy_sum8(t_" in sr and re.search(r"_c_\d+ < 4;", sr) and re.search(r"\* 4\) < 100\) \{", sr)
     assert "parpy_transpose_tile<float, 100, 1000>(" in sr and launch(sr)[0] == ("16", "2", "1", "256", "1", "1")
+    # the CSR entry point: decompression kernel, transposition, main kernel, in that order, in one host function
+    Cc = dict(C3, crows=crows3)
+    sc = compiles(parpy.print_compiled(W.sddmm_csr, [A3, B3, Cc, np.zeros_like(vals3), 1024, 1.5, 2.0],
+                                       opts_for({"N": parpy.threads(1024), "M": parpy.threads(32), "nnz": parpy.threads(n3)})))
+    host = sc[sc.index("// host side"):]
+    assert [m for m in re.findall(r"sddmm_csr_(\w+?)_\d+<<<", host)] == ["row", "transpose_B", "i"]
+    assert launch(sc)[0] == ("1", "1024", "1", "64", "1", "1")
     s = compiles(parpy.print_compiled(W.sddmm_decompress_csr, [crows, np.zeros_like(cols), 128],
                                       opts_for({"N": parpy.threads(128), "M": parpy.threads(64)})))
     assert launch(s) == [("1", "128", "1", "64", "1", "1")]

@@ -288,6 +288,23 @@ def test_sddmm(n, k, density, flags):
     assert np.abs(got - want).max() < 5e-4
 
 
+def test_sddmm_on_csr_mask_decompresses_rows_in_the_same_call():
+    """The reference's CSR entry (benchmarks/sddmm.py:29-61): the jitted decompression kernel is called from inside
+    the jitted SDDMM, with the reference's parallelisation (32 threads per row round up to one wavefront)."""
+    n, k = 1024, 96
+    A, B, crows, cols, vals = W.make_sddmm(n, k, 0.02)
+    nnz = len(cols)
+    C = {"crows": torch.from_numpy(crows).cuda(), "rows": torch.zeros(nnz, dtype=torch.int64, device="cuda"),
+         "cols": torch.from_numpy(cols).cuda(), "values": torch.from_numpy(vals).cuda(), "nnz": nnz}
+    D = torch.zeros(nnz, dtype=torch.float32, device="cuda")
+    W.sddmm_csr(torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda(), C, D, n, 1.5, 2.0,
+                opts=opts_for({"N": parpy.threads(n), "M": parpy.threads(32), "nnz": parpy.threads(nnz)}))
+    rows = oracle.csr_rows(crows)
+    assert np.array_equal(C["rows"].cpu().numpy(), rows)
+    want = oracle.sddmm(A, B, rows, cols, vals, alpha=1.5, beta=2.0)
+    assert np.allclose(D.cpu().numpy(), want, atol=1e-4, rtol=1e-5)
+
+
 # ---------------------------------------------------------------- surface behaviour
 def test_host_arrays_are_copied_back_and_device_arrays_are_shared():
     N = 1000
