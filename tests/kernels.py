@@ -152,3 +152,90 @@ def alias_maybe_same(a, b, N, M, steps):
             parpy.label('M')
             for j in range(M):
                 dst[i, j] = src[i, j] + float32(1.0)
+
+
+# ---------------------------------------------------------------- HMM forward pass out of small jitted pieces
+# The reference model's recurrence (test/test_forward.py:83-160, split per phase as in
+# benchmarks/forward.py:94-187) written with helper functions that return values: every score is an
+# expression call that the compiler inlines.  Operators are reached through a module alias.
+import parpy_amd.operators as ops
+
+
+@parpy.jit
+def shift_score(hmm, alpha, inst, state, j):
+    """Score of reaching `state` from its j-th shift predecessor (always in duration layer 0)."""
+    quarter = hmm["num_states"] // 64
+    kmers = hmm["num_states"] // 16
+    pred = ops.int32(j * quarter + (state // 4) % quarter)
+    return hmm["trans1"][pred % kmers, state % 4] + hmm["trans2"][state // kmers] + alpha[inst, pred]
+
+
+@parpy.jit
+def stay_score(hmm, alpha, inst, state):
+    """Score of reaching `state` by staying on its k-mer: from the next duration layer, or from itself in the last."""
+    kmers = hmm["num_states"] // 16
+    layer = state // kmers
+    pred = ops.int32(state)
+    p = hmm["gamma"]
+    if layer != 15:
+        pred = ops.int32(state + kmers)
+        p = ops.float32(0.0)
+        if layer == 14:
+            p = hmm["synthetic_248"]
+    return p + alpha[inst, pred]
+
+
+@parpy.jit
+def lse5(a, b, c, d, e):
+    m = ops.max(ops.max(ops.max(ops.max(a, b), c), d), e)
+    s = m + ops.log(ops.exp(a - m) + ops.exp(b - m) + ops.exp(c - m) + ops.exp(d - m) + ops.exp(e - m))
+    return ops.max(s, ops.float32(-ops.inf))
+
+
+@parpy.jit
+def pieces_init(hmm, seqs, alpha, inst):
+    o = seqs["data"][inst, 0]
+    parpy.label('state')
+    for state in range(hmm["num_states"]):
+        alpha[inst, state] = hmm["initial_prob"][state] + hmm["output_prob"][o, state % (hmm["num_states"] // 16)]
+
+
+@parpy.jit
+def pieces_step(hmm, seqs, alpha1, alpha2, inst, t):
+    src = alpha2
+    dst = alpha1
+    if t & 1:
+        src = alpha1
+        dst = alpha2
+    o = seqs["data"][inst, t]
+    parpy.label('state')
+    for state in range(hmm["num_states"]):
+        if t < seqs["lens"][inst]:
+            total = lse5(shift_score(hmm, src, inst, state, 0), shift_score(hmm, src, inst, state, 1),
+                         shift_score(hmm, src, inst, state, 2), shift_score(hmm, src, inst, state, 3),
+                         stay_score(hmm, src, inst, state))
+            dst[inst, state] = total + hmm["output_prob"][o, state % (hmm["num_states"] // 16)]
+        elif t == seqs["lens"][inst]:
+            dst[inst, state] = src[inst, state]
+
+
+@parpy.jit
+def pieces_total(hmm, seqs, result, alpha1, alpha2, inst):
+    alpha = alpha2
+    if seqs["maxlen"] & 1:
+        alpha = alpha1
+    parpy.label('state')
+    m = ops.max(alpha[inst, :], axis=0)
+    parpy.label('state')
+    s = ops.sum(ops.exp(alpha[inst, :] - m), axis=0)
+    result[inst] = m + ops.log(s)
+
+
+@parpy.jit
+def forward_in_pieces(hmm, seqs, alpha1, alpha2, result):
+    parpy.label('inst')
+    for inst in range(seqs["num_instances"]):
+        pieces_init(hmm, seqs, alpha1, inst)
+        for t in range(1, seqs["maxlen"]):
+            pieces_step(hmm, seqs, alpha1, alpha2, inst, t)
+        pieces_total(hmm, seqs, result, alpha1, alpha2, inst)

@@ -227,6 +227,21 @@ def test_reference_model_kernel_compiles(golden_dir):
         assert len(s) != 0
 
 
+def test_forward_written_with_value_returning_helpers_compiles_to_the_same_structure(golden_dir):
+    import os
+    import oracle
+    hmm, seqs = oracle.reference_model_tables(os.path.join(golden_dir, "hmm_3mer_model.npz"), os.path.join(golden_dir, "hmm_signals.npz"))
+    n, S = seqs["num_instances"], hmm["num_states"]
+    a = np.zeros((n, S), dtype=np.float32)
+    par = opts_for({'inst': parpy.threads(n), 'state': parpy.threads(512)})
+    pieces = compiles(parpy.print_compiled(K.forward_in_pieces, [hmm, seqs, a, a.copy(), np.zeros(n, dtype=np.float32)], par))
+    whole = compiles(parpy.print_compiled(W.forward_kernel, [hmm, seqs, a, a.copy(), np.zeros(n, dtype=np.float32)], par))
+    assert launch(pieces) == launch(whole) and len(launch(pieces)) == 1
+    for text in (pieces, whole):       # state vectors in LDS, five exponentials and one logarithm per state
+        body = text.split("extern \"C\" __global__")[1]
+        assert "lds_alpha1_" in body and "lds_alpha2_" in body
+
+
 def test_sddmm_kernels_compile():
     import oracle
     A, B, crows, cols, vals = W.make_sddmm(128, 16, 0.05)

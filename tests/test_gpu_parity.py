@@ -158,6 +158,22 @@ def test_forward_3mer_golden(golden_dir, threads):
     assert np.allclose(got, exp, atol=1e-5, rtol=1e-5), np.abs(got - exp).max()
 
 
+@pytest.mark.parametrize("threads", [512, 2048])
+def test_forward_written_with_value_returning_helpers(golden_dir, threads):
+    """The same recurrence assembled from jitted helpers that return values (every predecessor score and the
+    log-sum-exp are expression calls), operators reached through a module alias, reductions with `axis=0`:
+    after inlining it is the same computation and must reproduce the recorded log-likelihoods."""
+    hmm, seqs, exp = _golden(golden_dir, 3)
+    hd, sd = W.to_device(hmm), W.to_device(seqs)
+    n, S = seqs["num_instances"], hmm["num_states"]
+    a1 = torch.zeros((n, S), dtype=torch.float32, device="cuda")
+    a2 = torch.zeros_like(a1)
+    res = torch.zeros(n, dtype=torch.float32, device="cuda")
+    K.forward_in_pieces(hd, sd, a1, a2, res, opts=opts_for({'inst': parpy.threads(n), 'state': parpy.threads(threads)}))
+    got = res.cpu().numpy()
+    assert np.allclose(got, exp, atol=1e-5, rtol=1e-5), np.abs(got - exp).max()
+
+
 def test_forward_3mer_golden_unoptimised(golden_dir):
     hmm, seqs, exp = _golden(golden_dir, 3)
     got = _run_reference_model(hmm, seqs, 512, opt_lds_rows=False, opt_vectorize=False, opt_hoist_invariant=False,
