@@ -219,6 +219,59 @@ struct Pass {
     }
   };
 
+  // ================================================================ conditions no iteration changes
+  // A parallel loop whose whole body is `if (c) A else B`, with c the same for every iteration (it
+  // mentions neither the loop variable nor anything the body defines or assigns, and loads only from
+  // arrays the kernel never writes), becomes `if (c) { loop A } else { loop B }`.  The HMM step tests
+  // `t < lens[inst]` (and `t == lens[inst]` in the else branch) once per state; inside the unrolled
+  // loop that is a branch between any two states, which keeps the instructions of neighbouring
+  // states from being scheduled together.  Only tests with an else branch are rewritten: a plain
+  // `if (c) A` the device compiler unswitches by itself, and doing it here first was measured to
+  // cost 5 % on the single-layer HMM step (60.4 -> 63.4 ms; the 16-layer model gains 6 %).
+  Stmts hoist_uniform_conditions(const Stmts& ss) {
+    std::set<Name> params = param_names();
+    std::set<Name> written = written_arrays();
+    std::function<Stmts(const Stmts&)> walk = [&](const Stmts& in) -> Stmts {
+      Stmts out;
+      for (auto& s : in) {
+        bool done = false;
+        if (s->k == Stmt::For && s->map.k != GpuMap::None && s->body.size() == 1 && s->body[0]->k == Stmt::If && !s->body[0]->els.empty()) {
+          const S& test = s->body[0];
+          std::set<Name> local{s->id};
+          visit_stmts(s->body, [&](const S& c) {
+            if (c->k == Stmt::Def || c->k == Stmt::For) local.insert(c->id);
+            if (c->k == Stmt::Assign && c->dst->k == Expr::Var) local.insert(c->dst->name);
+          });
+          bool uniform = true;
+          visit_exprs(test->expr, [&](const E& x) {
+            if (x->k == Expr::Var && local.count(x->name)) uniform = false;
+            if (x->k == Expr::Index && !(x->args[0]->k == Expr::Var && params.count(x->args[0]->name) && !written.count(x->args[0]->name)))
+              uniform = false;
+            if (x->k == Expr::Call || x->k == Expr::Raw || x->k == Expr::RegElem || x->k == Expr::ThreadIdx) uniform = false;
+          });
+          if (uniform) {
+            auto loop_over = [&](const Stmts& body) {
+              auto n = clone(s);
+              n->body = body;
+              return walk({S(n)});
+            };
+            Stmts els;
+            if (!test->els.empty()) els = loop_over(test->els);
+            out.push_back(mk_if(test->expr, loop_over(test->body), els, test->i));
+            done = true;
+          }
+        }
+        if (done) continue;
+        auto r = clone(s);
+        r->body = walk(s->body);
+        r->els = walk(s->els);
+        out.push_back(r);
+      }
+      return out;
+    };
+    return walk(ss);
+  }
+
   void unswitch_aliases() {
     bool any = false;
     visit_stmts(k.body, [&](const S& s) { if (s->k == Stmt::Def && Unswitch::is_alias_type(s->ty)) any = true; });
@@ -1741,6 +1794,7 @@ void hip_optimize(Program& p, const Options& opts, NameGen& gen) {
     Pass pass(k, opts, gen);
     if (opts.opt_unswitch) pass.unswitch_aliases();
     if (opts.opt_mfma_sddmm) k.body = pass.mfma_dot(k.body);
+    if (opts.opt_unswitch_uniform) k.body = pass.hoist_uniform_conditions(k.body);
     if (opts.opt_lds_rows) pass.lds_rows();
     if (opts.opt_vectorize) k.body = pass.vectorize(k.body);
     int64_t budget = pass.reg_budget();

@@ -242,6 +242,25 @@ def test_forward_written_with_value_returning_helpers_compiles_to_the_same_struc
         assert "lds_alpha1_" in body and "lds_alpha2_" in body
 
 
+def test_tests_that_no_iteration_changes_move_out_of_the_state_loop(golden_dir):
+    """`if t < len: step elif t == len: copy` inside the state loop becomes two loops under the tests."""
+    import os
+    import oracle
+    hmm, seqs = oracle.reference_model_tables(os.path.join(golden_dir, "hmm_3mer_model.npz"), os.path.join(golden_dir, "hmm_signals.npz"))
+    n, S = seqs["num_instances"], hmm["num_states"]
+    a = np.zeros((n, S), dtype=np.float32)
+    args = [hmm, seqs, a, a.copy(), np.zeros(n, dtype=np.float32)]
+    par = {'inst': parpy.threads(n), 'state': parpy.threads(256)}
+    on = compiles(parpy.print_compiled(W.forward_kernel, args, opts_for(par))).split("extern \"C\" __global__")[1]
+    off = compiles(parpy.print_compiled(W.forward_kernel, args, opts_for(par, opt_unswitch_uniform=False))).split("extern \"C\" __global__")[1]
+    step = lambda text: text[text.index("for (int t_"):]
+    test = r"if \(t_\d+ < seqs_lens_\d+\[inst_\d+\]\) \{"
+    first_state = lambda text: re.search(r"int state_\w+ = ", step(text)).start()
+    # outside: the test comes before the states are enumerated; inside: after
+    assert re.search(test, step(on)).start() < first_state(on)
+    assert re.search(test, step(off)).start() > first_state(off)
+
+
 def test_sddmm_kernels_compile():
     import oracle
     A, B, crows, cols, vals = W.make_sddmm(128, 16, 0.05)
