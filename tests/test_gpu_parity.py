@@ -304,6 +304,24 @@ def test_sddmm(n, k, density, flags):
     assert np.abs(got - want).max() < 5e-4
 
 
+@pytest.mark.parametrize("k", [96, 50])
+def test_sddmm_in_double_precision(k):
+    """8-byte elements: two per 16-byte vector, sixteen per round of a lane group (k = 50: three rounds and a bit)."""
+    n = 512
+    A, B, crows, cols, vals = W.make_sddmm(n, k, 0.05)
+    A, B, vals = A.astype(np.float64), B.astype(np.float64), vals.astype(np.float64)
+    rows = oracle.csr_rows(crows)
+    nnz = len(cols)
+    C = {"rows": torch.from_numpy(rows).cuda(), "cols": torch.from_numpy(cols).cuda(), "values": torch.from_numpy(vals).cuda(), "nnz": nnz}
+    D = torch.zeros(nnz, dtype=torch.float64, device="cuda")
+    o = opts_for({"nnz": parpy.threads(nnz).tpb(256)})
+    W.sddmm_coo(torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda(), C, D, np.float64(1.5), np.float64(2.0), opts=o)
+    want = 1.5 * np.einsum("ij,ij->i", A[rows], B.T[cols]) + 2.0 * vals
+    assert np.allclose(D.cpu().numpy(), want, atol=1e-12, rtol=1e-12)
+    listing = parpy.print_compiled(W.sddmm_coo, [torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda(), C, D, np.float64(1.5), np.float64(2.0)], o)
+    assert "parpy_sum8(" in listing and "parpy_transpose_tile<double" in listing
+
+
 def test_sddmm_on_csr_mask_decompresses_rows_in_the_same_call():
     """The reference's CSR entry (benchmarks/sddmm.py:29-61): the jitted decompression kernel is called from inside
     the jitted SDDMM, with the reference's parallelisation (32 threads per row round up to one wavefront)."""
