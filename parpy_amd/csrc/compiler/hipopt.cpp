@@ -1611,10 +1611,12 @@ struct LaneSplit {
 
   // the sum loop: a sequential loop over [0, K) whose body is `acc = acc + e`, where acc is a scalar
   // variable or an array element that does not depend on d, and all d-dependent accesses are unit-stride
+  // (*vec = 0 stands for the second form: bounds that are data, as in a CSR row -- then lane g of a group takes
+  // the elements lo+g, lo+g+8, ... one at a time, since nothing is known about where the row starts.)
   bool sum_loop(const S& s, int* vec, E* term_out) {
-    if (!(s->k == Stmt::For && s->map.k == GpuMap::None && !s->unroll && s->step == 1 && s->lo->k == Expr::Int && s->lo->iv == 0 &&
-          s->hi->k == Expr::Int && s->body.size() == 1))
-      return false;
+    if (!(s->k == Stmt::For && s->map.k == GpuMap::None && !s->unroll && s->step == 1 && s->body.size() == 1)) return false;
+    const bool fixed = s->lo->k == Expr::Int && s->lo->iv == 0 && s->hi->k == Expr::Int;
+    if (!fixed && s->lo->k == Expr::Int && s->hi->k == Expr::Int) return false;  // constant bounds that do not start at 0: not handled
     const S& a = s->body[0];
     if (a->k != Stmt::Assign) return false;
     const E& acc = a->dst;
@@ -1628,7 +1630,7 @@ struct LaneSplit {
     else if (expr_eq(r, acc)) term = l;
     if (!term) return false;
     const Name& acc_name = scalar_acc ? acc->name : acc->args[0]->name;
-    if (mentions(term, acc_name)) return false;
+    if (mentions(term, acc_name) || mentions(s->lo, acc_name) || mentions(s->hi, acc_name)) return false;
     int v = 0, loads = 0;
     bool ok = true;
     visit_exprs(term, [&](const E& x) {
@@ -1636,14 +1638,15 @@ struct LaneSplit {
       if (x->k != Expr::Index) return;
       if (!mentions(x->args[1], s->id)) return;
       E rest;
-      if (!affine_unit(x->args[1], s->id, &rest)) { ok = false; return; }
+      if (!affine_unit(x->args[1], s->id, &rest)) { if (fixed) ok = false; return; }  // (a gather `x[cols[d]]` is fine lane by lane)
       int w = elem_bytes(x->ty.sz) == 4 ? 4 : elem_bytes(x->ty.sz) == 8 ? 2 : 0;
       if (w == 0) { ok = false; return; }
       v = v == 0 ? w : std::min(v, w);
       ++loads;
     });
-    if (!ok || loads < 1 || s->hi->iv % v != 0 || s->hi->iv < 2 * v * G) return false;  // whole vectors, and enough of them
-    *vec = v;
+    if (!ok || loads < 1) return false;
+    if (fixed && (s->hi->iv % v != 0 || s->hi->iv < 2 * v * G)) return false;  // whole vectors, and enough of them
+    *vec = fixed ? v : 0;
     *term_out = term;
     return true;
   }
@@ -1713,6 +1716,14 @@ struct LaneSplit {
       body.push_back(mk_def(tn, acc->ty, mk_float(0.0, acc->ty.sz), loop->i));
       t = mk_var(tn, acc->ty);
     }
+    if (vec == 0) {
+      // bounds that are data: for (d = lo + g; d < hi; d += G) t += term
+      auto strided = clone(loop);
+      strided->lo = mk_binop(BinOp::Add, loop->lo, gv, ity);
+      strided->step = G;
+      strided->body = {mk_assign(t, mk_binop(BinOp::Add, t, term, t->ty), loop->i)};
+      body.push_back(strided);
+    } else {
     // d = (d0 * G + g) * V + u
     E d = mk_binop(BinOp::Add,
                    mk_binop(BinOp::Mul, mk_binop(BinOp::Add, mk_binop(BinOp::Mul, mk_var(d0, ity), mk_int(G, isz), ity), gv, ity),
@@ -1737,6 +1748,7 @@ struct LaneSplit {
       outer->body = {mk_if(mk_binop(BinOp::Lt, base, mk_int(K, isz), Type::scalar(ElemSize::Bool)), {S(inner)}, {})};
     }
     body.push_back(outer);
+    }
     body.push_back(mk_assign(t, mk_raw("parpy_sum8(" + t->name.str() + ")", t->ty)));
     Stmts stores;
     if (elem_acc) {

@@ -3,6 +3,8 @@ and run against NumPy (GPU part): symmetric rank-k update with a triangular iter
 (test/test_syrk.py), CSR SpMV and SpMM with data-dependent loop bounds (test/test_spmv.py,
 test/test_spmm.py), nested loops with different inner thread counts (test/test_sync.py:57-92),
 a Jacobi stencil on shifted slices and matrix products on slices (test/test_slicing.py)."""
+import re
+
 import numpy as np
 import pytest
 
@@ -175,6 +177,31 @@ def test_spmv(p):
     y = np.zeros(256, dtype=np.float32)
     parpy.jit(spmv)(A, x, y, opts=opts_for(p))
     assert np.allclose(y, dense.astype(np.float64) @ x, atol=1e-4)
+
+
+def test_spmv_with_one_thread_per_row_shares_rows_among_eight_lanes():
+    """Bounds that are data (a CSR row): lane g of a group of eight takes the elements lo+g, lo+g+8, ...;
+    the gather x[cols[i]] goes lane by lane, the partial sums meet in three cross-lane steps."""
+    A, _ = random_csr(256, 4096, 0.01, 1)
+    args = [A, np.zeros(4096, dtype=np.float32), np.zeros(256, dtype=np.float32)]
+    s = compiles(parpy.print_compiled(spmv, args, opts_for({"row": parpy.threads(256)})))
+    assert re.search(r"i_\d+ \+= 8\)", s) and "= parpy_sum8(" in s and "<<<dim3(8, 1, 1), dim3(256, 1, 1)" in s
+    s = compiles(parpy.print_compiled(spmv, args, opts_for({"row": parpy.threads(256)}, opt_lane_split=False)))
+    assert "= parpy_sum8(" not in s and "<<<dim3(1, 1, 1), dim3(256, 1, 1)" in s
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("rows,density", [(5000, 0.002), (300, 0.05), (64, 0.3)])
+def test_spmv_with_one_thread_per_row_on_ragged_rows(rows, density):
+    A, dense = random_csr(rows, 2048, density, rows)
+    lens = np.diff(A["rows"])
+    assert lens.min() == 0 or rows < 1000          # the big case has empty rows
+    x = np.random.default_rng(7).standard_normal(2048).astype(np.float32)
+    want = dense.astype(np.float64) @ x
+    for split in (True, False):
+        y = np.zeros(rows, dtype=np.float32)
+        parpy.jit(spmv)(A, x, y, opts=opts_for({"row": parpy.threads(rows)}, opt_lane_split=split))
+        assert np.allclose(y, want, atol=1e-4), (rows, split)
 
 
 @pytest.mark.gpu
