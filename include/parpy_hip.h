@@ -69,7 +69,10 @@ int32_t parpy_hip_plan_create(void* module, const char* plan_text, void** plan);
 
 /* Run the plan: `args` are the flattened pointer arguments in call order
  * (dict fields sorted by key, python/parpy/compile.py:142-146); scalars were
- * folded into the code at compile time.  Returns 0 or non-zero. */
+ * folded into the code at compile time.  Returns 0 or non-zero.  A plan holds
+ * the state of its host loops and its device temporaries: runs of one plan
+ * from several host threads take turns (different plans run concurrently);
+ * the error message is per thread. */
 int32_t parpy_hip_plan_run(void* plan, void* const* args, int32_t nargs);
 
 /* Same as parpy_hip_plan_run, bracketed by HIP events recorded on the null
