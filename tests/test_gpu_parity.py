@@ -90,6 +90,19 @@ def test_one_thread_per_row_inside_one_workgroup(rows, cols):
         assert np.allclose(out, x.astype(np.float64).sum(axis=1), atol=1e-4, rtol=1e-5), (rows, cols, split)
 
 
+def test_rows_of_a_matrix_with_more_than_2_to_31_elements():
+    """3.2e9 elements (12.8 GB): flat indices need 64 bits even though every loop variable fits in 32."""
+    N, M = 100, 32_000_000
+    x = torch.full((N, M), 0.5, dtype=torch.float32, device="cuda")
+    x[N - 1, M - 1] = 2.5                      # the very last element, at flat index 3 199 999 999
+    out = torch.zeros(N, dtype=torch.float32, device="cuda")
+    parpy.jit(K.sum_rows)(x, out, N, opts=opts_for({'outer': parpy.threads(N), 'inner': parpy.threads(1024)}))
+    want = torch.full((N,), 0.5 * M, dtype=torch.float32, device="cuda")
+    want[N - 1] += 2.0
+    assert torch.equal(out, want)              # sums of halves below 2^24 are exact in any order
+    del x
+
+
 @pytest.mark.parametrize("threads", [64, 2048])
 def test_strided_reduction(threads):
     N, M = 10, 4096
