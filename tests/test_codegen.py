@@ -132,6 +132,19 @@ def test_register_budget_counts_what_is_live_at_once():
     assert "float row_" not in s.split("extern \"C\" __global__")[1]
 
 
+def test_one_element_per_thread_becomes_four_on_large_element_wise_launches():
+    n = 1 << 24
+    x = np.zeros(n, dtype=np.float32)
+    s = compiles(parpy.print_compiled(K.axpy, [2.0, x, x, x.copy(), n], opts_for({'N': parpy.threads(n)})))
+    assert launch(s) == [(str(n // 4 // 1024), "1", "1", "1024", "1", "1")] and re.search(r"_u_\d+ < 4;", s)
+    # a launch that would leave CUs short of threads keeps one element per thread; so does an unaligned argument
+    m = 1 << 15
+    s = compiles(parpy.print_compiled(K.axpy, [2.0, x[:m], x[:m], x[:m].copy(), m], opts_for({'N': parpy.threads(m)})))
+    assert launch(s) == [(str(m // 1024), "1", "1", "1024", "1", "1")]
+    s = compiles(parpy.print_compiled(K.axpy, [2.0, x, x, x.copy(), n], opts_for({'N': parpy.threads(n)}, assume_aligned=False)))
+    assert launch(s) == [(str(n // 1024), "1", "1", "1024", "1", "1")] and not re.search(r"_u_\d+ < 4;", s.split("extern \"C\" __global__")[1])
+
+
 def test_grid_wide_loop_is_vectorised_when_no_block_is_partial():
     n = 1 << 20
     x = np.zeros(n, dtype=np.float32)
