@@ -31,6 +31,11 @@ def compiles(listing, opts=None):
     return listing
 
 
+def elem(a):
+    """Regular expression for the start of an element access of array `a` (subscript or 32-bit offset form)."""
+    return r"(?:%s_\d+\[|parpy_at\(%s_\d+, )" % (a, a)
+
+
 def launch(listing):
     return re.findall(r"<<<dim3\((\d+), (\d+), (\d+)\), dim3\((\d+), (\d+), (\d+)\)", listing)
 
@@ -109,12 +114,12 @@ def test_softmax_is_one_kernel_and_row_resident():
     assert launch(s) == [("1", "256", "1", "1024", "1", "1")]
     body = s.split("extern \"C\" __global__")[1]
     # register caching: x is read from memory once and out is written once
-    assert len(re.findall(r"= x_\d+\[", body)) == 1 and len(re.findall(r"&out_\d+\[", body)) == 1
+    assert len(re.findall(r"= " + elem("x"), body)) == 1 and len(re.findall(r"&" + elem("out"), body)) == 1
     # the result is streamed out: nothing reads it again
     assert "__builtin_nontemporal_store(" in body
     s0 = compiles(parpy.print_compiled(W.softmax, [x, N, M, x.copy()],
                                        opts_for({'N': parpy.threads(N), 'M': parpy.threads(1024)}, opt_reg_cache=False)))
-    assert len(re.findall(r"x_\d+\[", s0.split("extern \"C\" __global__")[1])) >= 2
+    assert len(re.findall(elem("x"), s0.split("extern \"C\" __global__")[1])) >= 2
 
 
 def test_register_budget_counts_what_is_live_at_once():
@@ -124,7 +129,7 @@ def test_register_budget_counts_what_is_live_at_once():
     x = np.zeros((N, M), dtype=np.float32)
     s = compiles(parpy.print_compiled(W.softmax, [x, N, M, x.copy()], opts_for({'N': parpy.threads(N), 'M': parpy.threads(1024)})))
     body = s.split("extern \"C\" __global__")[1]
-    assert len(re.findall(r"= x_\d+\[", body)) == 1 and len(re.findall(r"&out_\d+\[", body)) == 1
+    assert len(re.findall(r"= " + elem("x"), body)) == 1 and len(re.findall(r"&" + elem("out"), body)) == 1
     assert "float row_x_" in body and "float row_out_" in body
     # twice the row: nothing fits any more and the four statements go through memory
     x = np.zeros((N, 2 * M), dtype=np.float32)
@@ -179,7 +184,7 @@ def test_softmax_rows_stay_in_registers_when_the_block_does_not_divide_them():
     x = np.zeros((N, M), dtype=np.float32)
     s = compiles(parpy.print_compiled(W.softmax, [x, N, M, x.copy()], opts_for({'N': parpy.threads(N), 'M': parpy.threads(64)})))
     body = s.split("extern \"C\" __global__")[1]
-    assert len(re.findall(r"= x_\d+\[", body)) == 1 and len(re.findall(r"&out_\d+\[", body)) == 1
+    assert len(re.findall(r"= " + elem("x"), body)) == 1 and len(re.findall(r"&" + elem("out"), body)) == 1
     assert len(re.findall(r"if \(\w+ < 250\) \{", body)) == 4
 
 
@@ -267,7 +272,7 @@ def test_tests_that_no_iteration_changes_move_out_of_the_state_loop(golden_dir):
     on = compiles(parpy.print_compiled(W.forward_kernel, args, opts_for(par))).split("extern \"C\" __global__")[1]
     off = compiles(parpy.print_compiled(W.forward_kernel, args, opts_for(par, opt_unswitch_uniform=False))).split("extern \"C\" __global__")[1]
     step = lambda text: text[text.index("for (int t_"):]
-    test = r"if \(t_\d+ < seqs_lens_\d+\[inst_\d+\]\) \{"
+    test = r"if \(t_\d+ < " + elem("seqs_lens")
     first_state = lambda text: re.search(r"int state_\w+ = ", step(text)).start()
     # outside: the test comes before the states are enumerated; inside: after
     assert re.search(test, step(on)).start() < first_state(on)
