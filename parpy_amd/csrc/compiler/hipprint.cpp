@@ -392,16 +392,29 @@ struct DevicePrinter {
         // [0, extent) while this address is computed, which lets gathered indices (loaded from memory,
         // so of unknown range) take part in 32-bit address arithmetic.
         std::vector<Name> assumed;
+        std::vector<std::pair<Name, Interval>> narrowed;
         for (size_t d = 0; d < e->dim_idx.size() && d < e->dim_shape.size(); ++d) {
-          const E& x = e->dim_idx[d];
-          if (x->k == Expr::Var && is_i64(x) && !ranges.count(x->name)) {
-            Interval r;
-            r.known = true;
-            r.lo = 0;
-            r.hi = e->dim_shape[d] - 1;
-            ranges[x->name] = r;
+          E x = e->dim_idx[d];
+          while (x->k == Expr::Convert && x->ty.is_scalar() && is_int(x->ty.sz) && x->args[0]->ty.is_scalar() && is_int(x->args[0]->ty.sz) &&
+                 elem_bytes(x->ty.sz) >= elem_bytes(x->args[0]->ty.sz))
+            x = x->args[0];  // (a narrow index widened: same value)
+          if (!(x->k == Expr::Var && x->ty.is_scalar() && is_int(x->ty.sz))) continue;
+          Interval r;
+          r.known = true;
+          r.lo = 0;
+          r.hi = e->dim_shape[d] - 1;
+          auto it = ranges.find(x->name);
+          if (it == ranges.end()) {
             assumed.push_back(x->name);
+          } else {
+            // a range that is only the variable's type (an int8 observation: -128..127) is cut to the extent
+            if (!it->second.known || (it->second.lo >= 0 && it->second.hi <= r.hi)) continue;
+            narrowed.push_back({x->name, it->second});
+            r.lo = std::max(r.lo, it->second.lo);
+            r.hi = std::min(r.hi, it->second.hi);
+            if (r.lo > r.hi) { narrowed.pop_back(); continue; }
           }
+          ranges[x->name] = r;
         }
         std::string out = pexpr(e->args[0]) + "[" + pexpr(e->args[1]) + "]";
         if (opts.opt_offset32 && e->args[0]->ty.mem != Mem::LDS) {
@@ -415,6 +428,7 @@ struct DevicePrinter {
             out = "parpy_at(" + pexpr(e->args[0]) + ", (unsigned)(" + pexpr(e->args[1]) + "))";
         }
         for (auto& n : assumed) ranges.erase(n);
+        for (auto& kv : narrowed) ranges[kv.first] = kv.second;
         return out;
       }
       case Expr::AddrOf: return "(&" + pexpr(e->args[0]) + "[" + pexpr(e->args[1]) + "])";
