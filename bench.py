@@ -121,7 +121,7 @@ def bench_hmm_ref(args, torch, parpy, W):
 def bench_rowsum(args, torch, parpy, W):
     import numpy as np
     N, M = 1024, 65536
-    args.inner_threads = args.inner_threads or 256   # 4 workgroups per CU overlap their load and reduce phases
+    args.inner_threads = args.inner_threads or 1024  # one full workgroup per row (any choice from 64 up measures within 5 %)
     x = W.make_rowsum(N, M)
     xd = torch.from_numpy(x).cuda()
     out = torch.zeros(N, dtype=torch.float32, device="cuda")
