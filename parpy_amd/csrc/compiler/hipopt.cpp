@@ -15,7 +15,20 @@
 //                   the thread's own iteration, inside a sequential loop, are
 //                   done once before the loop into per-thread registers;
 //   reg_cache       array sections that a thread alone reads and writes across
-//                   consecutive parallel loops stay in registers in between.
+//                   consecutive parallel loops stay in registers in between;
+//   hoist_uniform_conditions
+//                   `for x: if (c) A else B` with c the same for every x becomes
+//                   `if (c) for x: A else for x: B`;
+//   drop_barriers   barriers between regions that share no written array go.
+//
+// Three rewrites work on the whole program because they change a launch:
+//   GatherTranspose column gathers X[d, c] over an innermost sequential d read a
+//                   transposed copy made by a tiled kernel in front of the launch;
+//   LaneSplit       eight adjacent lanes share one iteration's sequential sum
+//                   (constant bounds: 16-byte pieces of each line; bounds that
+//                   are data, as in a CSR row: one element each, stride 8);
+//   Coarsen         a large element-wise launch with one element per thread is
+//                   cut to a quarter so that vectorize gives each thread four.
 //
 // Each pass can be switched off through the options (tests compare the
 // results with and without them).
