@@ -8,7 +8,7 @@ HIP backend -- nothing here calls a hand-written kernel.
 import numpy as np
 
 import parpy_amd as parpy
-from parpy_amd.operators import exp, float32, inf, int16, int32, log, max, sum
+from parpy_amd.operators import exp, float32, inf, int32, log, max, sum
 
 
 # ---------------------------------------------------------------- reductions / softmax
