@@ -249,7 +249,7 @@ def _profiled_traffic(name):
 
 
 def _apply_opt_flags(opts, args):
-    for name in ("opt_vectorize", "opt_lds_rows", "opt_reg_cache", "opt_hoist_invariant", "opt_narrow_index", "opt_unswitch", "opt_gather_transpose", "opt_nontemporal", "opt_lane_split", "opt_drop_barriers", "opt_unswitch_uniform", "opt_offset32", "opt_noalias_scopes", "opt_mfma_sddmm"):
+    for name in ("opt_vectorize", "opt_lds_rows", "opt_reg_cache", "opt_hoist_invariant", "opt_narrow_index", "opt_unswitch", "opt_gather_transpose", "opt_nontemporal", "opt_lane_split", "opt_drop_barriers", "opt_unswitch_uniform", "opt_offset32", "opt_if_convert", "opt_noalias_scopes", "opt_mfma_sddmm"):
         v = getattr(args, name)
         if v is not None:
             setattr(opts, name, bool(v))
@@ -269,7 +269,7 @@ def main():
     ap.add_argument("--tpb", type=int, default=256)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-steps", type=int, default=0, help="samples per read for the HMM CPU baseline")
-    for name in ("opt_vectorize", "opt_lds_rows", "opt_reg_cache", "opt_hoist_invariant", "opt_narrow_index", "opt_unswitch", "opt_gather_transpose", "opt_nontemporal", "opt_lane_split", "opt_drop_barriers", "opt_unswitch_uniform", "opt_offset32", "opt_noalias_scopes", "opt_mfma_sddmm"):
+    for name in ("opt_vectorize", "opt_lds_rows", "opt_reg_cache", "opt_hoist_invariant", "opt_narrow_index", "opt_unswitch", "opt_gather_transpose", "opt_nontemporal", "opt_lane_split", "opt_drop_barriers", "opt_unswitch_uniform", "opt_offset32", "opt_if_convert", "opt_noalias_scopes", "opt_mfma_sddmm"):
         ap.add_argument("--" + name.replace("_", "-"), dest=name, type=int, default=None)
     ap.add_argument("--reg-budget", type=int, default=0)
     args = ap.parse_args()
@@ -300,7 +300,7 @@ def main():
     else:
         r = bench_sddmm(args, torch, parpy, W)
     default_cfg = not any(getattr(args, n) is not None for n in ("opt_vectorize", "opt_lds_rows", "opt_reg_cache",
-                                                                 "opt_hoist_invariant", "opt_narrow_index", "opt_unswitch", "opt_gather_transpose", "opt_nontemporal", "opt_lane_split", "opt_drop_barriers", "opt_unswitch_uniform", "opt_offset32", "opt_noalias_scopes", "opt_mfma_sddmm"))
+                                                                 "opt_hoist_invariant", "opt_narrow_index", "opt_unswitch", "opt_gather_transpose", "opt_nontemporal", "opt_lane_split", "opt_drop_barriers", "opt_unswitch_uniform", "opt_offset32", "opt_if_convert", "opt_noalias_scopes", "opt_mfma_sddmm"))
     if default_cfg and not args.reg_budget:
         r["roofline"]["traffic"] = _profiled_traffic(args.workload)
     r.update({"n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "scaling": "weak", "vs_baseline": None,

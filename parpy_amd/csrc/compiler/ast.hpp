@@ -378,6 +378,7 @@ struct Options {  // src/option.rs:14-108
   bool opt_noalias_scopes = false; // aliases that always name different arrays are declared not to alias; measured slower on the HMM kernels: opt-in
   bool opt_unswitch_uniform = true; // `for x: if (uniform) A else B` -> `if (uniform) for x: A else for x: B`
   bool opt_offset32 = true;         // global elements at base + 32-bit byte offset when the offset provably fits
+  bool opt_if_convert = true;       // branches that only assign cheap scalar values become selects
   bool opt_drop_barriers = true;   // barriers between regions that share no written array are removed
   bool opt_lane_split = true;      // eight lanes share each long per-thread dot product
   bool opt_nontemporal = true;   // non-temporal stores to arrays a kernel only writes

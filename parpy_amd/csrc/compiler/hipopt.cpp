@@ -285,6 +285,92 @@ struct Pass {
     return walk(ss);
   }
 
+  // ================================================================ branches that only pick values
+  // `if (c) { x = a; y = b } else { x = d }` where every statement assigns a scalar variable a value that
+  // is free to compute either way (no memory access, no call, no division) becomes
+  // `x = c ? a : d; y = c ? b : y`.  The HMM step picks the predecessor and the score of the stay
+  // transition with an if / elif / else over the duration layer of the state; as branches these were
+  // eight execution-mask regions per sixteen states in the unrolled loop.
+  Stmts if_convert(const Stmts& ss) {
+    // variables that stand for a non-zero integer constant (`num_kmers = 1024`): dividing by them is safe to do early
+    std::set<Name> reassigned, nonzero_const;
+    visit_stmts(k.body, [&](const S& st) { if (st->k == Stmt::Assign && st->dst->k == Expr::Var) reassigned.insert(st->dst->name); });
+    visit_stmts(k.body, [&](const S& st) {
+      if (st->k == Stmt::Def && st->expr && st->expr->k == Expr::Int && st->expr->iv != 0 && !reassigned.count(st->id)) nonzero_const.insert(st->id);
+    });
+    return if_convert(ss, nonzero_const);
+  }
+
+  Stmts if_convert(const Stmts& ss, const std::set<Name>& nonzero_const) {
+    auto cheap = [&](const E& e) {
+      bool ok = true;
+      visit_exprs(e, [&](const E& x) {
+        if (x->k == Expr::Index || x->k == Expr::AddrOf || x->k == Expr::Call || x->k == Expr::Raw || x->k == Expr::RegElem) ok = false;
+        if (x->k == Expr::BinOpE && (x->bop == BinOp::Div || x->bop == BinOp::FloorDiv || x->bop == BinOp::Rem) &&
+            !((x->args[1]->k == Expr::Int && x->args[1]->iv != 0) || (x->args[1]->k == Expr::Var && nonzero_const.count(x->args[1]->name))))
+          ok = false;
+        if (x->k == Expr::BinOpE && x->bop == BinOp::Pow) ok = false;
+      });
+      return ok;
+    };
+    // a branch qualifies if it is a list of assignments to distinct scalar variables, none of which reads a
+    // variable assigned in the same `if` (either branch): then the order of the selects does not matter
+    auto values = [&](const Stmts& branch, std::vector<std::pair<E, E>>* out) {
+      for (auto& st : branch) {
+        if (st->k != Stmt::Assign || st->dst->k != Expr::Var || !st->dst->ty.is_scalar() || !cheap(st->expr)) return false;
+        for (auto& kv : *out)
+          if (kv.first->name == st->dst->name) return false;
+        out->push_back({st->dst, st->expr});
+      }
+      return true;
+    };
+    Stmts out;
+    for (auto& s : ss) {
+      auto r = clone(s);
+      r->body = if_convert(s->body, nonzero_const);
+      r->els = if_convert(s->els, nonzero_const);
+      bool done = false;
+      // (the test itself is evaluated once, as before, so it may read memory)
+      bool plain_test = true;
+      if (r->k == Stmt::If)
+        visit_exprs(r->expr, [&](const E& x) { if (x->k == Expr::Call || x->k == Expr::Raw || x->k == Expr::AddrOf) plain_test = false; });
+      if (r->k == Stmt::If && plain_test && !(r->body.empty() && r->els.empty())) {
+        std::vector<std::pair<E, E>> thn, els;
+        if (values(r->body, &thn) && values(r->els, &els)) {
+          std::set<Name> assigned;
+          for (auto& kv : thn) assigned.insert(kv.first->name);
+          for (auto& kv : els) assigned.insert(kv.first->name);
+          bool independent = true;
+          auto reads_assigned = [&](const E& e) { visit_exprs(e, [&](const E& x) { if (x->k == Expr::Var && assigned.count(x->name)) independent = false; }); };
+          for (auto& kv : thn) reads_assigned(kv.second);
+          for (auto& kv : els) reads_assigned(kv.second);
+          reads_assigned(r->expr);
+          if (independent && assigned.size() <= 4) {
+            E test = r->expr;
+            if (!cheap(test)) {   // reads memory: evaluated once, under a name (a cheap test is repeated, which lets a chain of elifs collapse)
+              Name c = gen.fresh("pick");
+              out.push_back(mk_def(c, Type::scalar(ElemSize::Bool), test, r->i));
+              test = mk_var(c, Type::scalar(ElemSize::Bool), r->i);
+            }
+            for (auto& name : assigned) {
+              E var, a, b;
+              for (auto& kv : thn) if (kv.first->name == name) { var = kv.first; a = kv.second; }
+              for (auto& kv : els) if (kv.first->name == name) { var = kv.first; b = kv.second; }
+              if (!a) a = var;
+              if (!b) b = var;
+              if (a->ty.sz != var->ty.sz) a = fold_expr(mk_convert(a, var->ty.sz));
+              if (b->ty.sz != var->ty.sz) b = fold_expr(mk_convert(b, var->ty.sz));
+              out.push_back(mk_assign(var, mk_ifexpr(test, a, b, var->ty, r->i), r->i));
+            }
+            done = true;
+          }
+        }
+      }
+      if (!done) out.push_back(r);
+    }
+    return out;
+  }
+
   void unswitch_aliases() {
     bool any = false;
     visit_stmts(k.body, [&](const S& s) { if (s->k == Stmt::Def && Unswitch::is_alias_type(s->ty)) any = true; });
@@ -1875,6 +1961,7 @@ void hip_optimize(Program& p, const Options& opts, NameGen& gen) {
     if (opts.opt_unswitch) pass.unswitch_aliases();
     if (opts.opt_mfma_sddmm) k.body = pass.mfma_dot(k.body);
     if (opts.opt_unswitch_uniform) k.body = pass.hoist_uniform_conditions(k.body);
+    if (opts.opt_if_convert) k.body = pass.if_convert(k.body);
     if (opts.opt_lds_rows) pass.lds_rows();
     if (opts.opt_vectorize) k.body = pass.vectorize(k.body);
     int64_t budget = pass.reg_budget();

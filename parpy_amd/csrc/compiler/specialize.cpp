@@ -87,6 +87,7 @@ Options parse_options(const std::string& sexpr) {
     else if (h == "opt_drop_barriers") o.opt_drop_barriers = flag();
     else if (h == "opt_unswitch_uniform") o.opt_unswitch_uniform = flag();
     else if (h == "opt_offset32") o.opt_offset32 = flag();
+    else if (h == "opt_if_convert") o.opt_if_convert = flag();
     else if (h == "opt_noalias_scopes") o.opt_noalias_scopes = flag();
     else if (h == "opt_gather_transpose") o.opt_gather_transpose = flag();
     else if (h == "reg_budget") o.reg_budget = f->at(1)->as_int();

@@ -252,6 +252,7 @@ class CompileOptions:
         'opt_drop_barriers': None,
         'opt_unswitch_uniform': None,
         'opt_offset32': None,
+        'opt_if_convert': None,
         'opt_noalias_scopes': None,
         'reg_budget': None,   # registers per thread the caching passes may claim (None: by block size)
         'assume_aligned': None,   # set by the driver: False when an array argument is not 16-byte aligned

@@ -469,3 +469,45 @@ def test_random_expressions_on_device(kind, dtype):
         else:
             ok = np.array_equal(got, want)
         assert ok, (expr, got[:4], want[:4])
+
+
+# ---------------------------------------------------------------- branches that only pick values
+def pick_values(x, y, out, N):
+    parpy.label('N')
+    for i in range(N):
+        a = ops.float32(0.0)
+        k = 0
+        if x[i] > 0.5:
+            a = x[i] * 2.0
+            k = i % 7
+        elif y[i] < 0.0:
+            a = ops.float32(-1.0)
+        else:
+            k = i // 3
+        b = ops.float32(1.0)
+        if y[i] > 0.25:            # one-sided: b keeps its value otherwise
+            b = ops.float32(3.0)
+        out[i] = a + b + ops.float32(k)
+
+
+def test_branches_that_only_assign_scalars_become_selects():
+    N = 256
+    x, y, out = np.zeros(N, dtype=np.float32), np.zeros(N, dtype=np.int32), np.zeros(N, dtype=np.float32)
+    on = compiles(parpy.print_compiled(pick_values, [x, y.astype(np.float32), out, N], opts_for({'N': parpy.threads(N)})))
+    off = compiles(parpy.print_compiled(pick_values, [x, y.astype(np.float32), out, N], opts_for({'N': parpy.threads(N)}, opt_if_convert=False)))
+    body = lambda s: s.split('extern "C" __global__')[1]
+    # the branch that loads x[i] in its value stays a branch (a load is not free to do either way); the others go
+    assert body(off).count("if (") - body(on).count("if (") >= 2 and " ? " in body(on)
+
+
+@pytest.mark.gpu
+def test_branches_that_only_assign_scalars_keep_their_meaning_as_selects():
+    rng = np.random.default_rng(12)
+    N = 1000
+    x, y = rng.uniform(0, 1, N).astype(np.float32), rng.uniform(-1, 1, N).astype(np.float32)
+    want = np.zeros(N, dtype=np.float32)
+    pick_values(x, y, want, N)
+    for flag in (True, False):
+        got = np.zeros(N, dtype=np.float32)
+        parpy.jit(pick_values)(x, y, got, N, opts=opts_for({'N': parpy.threads(N)}, opt_if_convert=flag))
+        assert np.allclose(got, want, rtol=1e-6), flag
