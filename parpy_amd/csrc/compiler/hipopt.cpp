@@ -914,6 +914,60 @@ struct Pass {
               if (h.load->k != Expr::Index) *budget -= is.slots * std::max(1, elem_bytes(h.sz) / 4);
             hoisted = live;
           }
+          // Values picked by tests on the iteration alone (`layer == 15 ? gamma : layer == 14 ? tail : 0`, and the
+          // predecessor index chosen the same way) are invariant as well: a compare and a select per test and
+          // step otherwise.  The largest such expressions move into a register per iteration.
+          {
+                        std::function<bool(const E&)> has_select = [&](const E& e) {
+              bool f = false;
+              visit_exprs(e, [&](const E& x) { if (x->k == Expr::IfExpr) f = true; });
+              return f;
+            };
+            std::function<E(const E&)> pick = [&](const E& e) -> E {
+              if (!e) return e;
+              if (e->k == Expr::IfExpr && e->ty.is_scalar() && elem_bytes(e->ty.sz) <= 4 && has_select(e)) {
+                E v = fold_expr(subst_vars(e, defs));
+                bool pure = true;
+                visit_exprs(v, [&](const E& x) {
+                  if (x->k == Expr::Var && !iter_vars.count(x->name)) pure = false;
+                  if (x->k == Expr::Index || x->k == Expr::RegElem || x->k == Expr::ThreadIdx || x->k == Expr::BlockIdx || x->k == Expr::Call ||
+                      x->k == Expr::Raw || x->k == Expr::AddrOf)
+                    pure = false;
+                });
+                int64_t cost = is.slots;
+                if (pure && *budget >= cost) {
+                  for (auto& h : hoisted)
+                    if (h.load->k != Expr::Index && expr_eq(h.load, v)) {
+                      auto re = std::make_shared<Expr>();
+                      re->k = Expr::RegElem; re->ty = e->ty; re->name = h.reg; re->args = {is.slot};
+                      return re;
+                    }
+                  *budget -= cost;
+                  Hoisted h;
+                  h.load = v;
+                  h.reg = gen.fresh("inv_pick");
+                  h.sz = e->ty.sz;
+                  hoisted.push_back(h);
+                  auto re = std::make_shared<Expr>();
+                  re->k = Expr::RegElem; re->ty = e->ty; re->name = h.reg; re->args = {is.slot};
+                  return re;
+                }
+              }
+              return map_children(e, pick);
+            };
+            std::function<Stmts(const Stmts&)> walk_picks = [&](const Stmts& b) {
+              Stmts o;
+              for (auto& c : b) {
+                auto nn = clone(c);
+                if (c->k == Stmt::Assign || c->k == Stmt::Def) nn->expr = pick(c->expr);
+                nn->body = walk_picks(c->body);
+                nn->els = walk_picks(c->els);
+                o.push_back(nn);
+              }
+              return o;
+            };
+            nbody = walk_picks(nbody);
+          }
           // loop nest that fills the registers, with the same thread mapping
           std::map<Name, Name> ren;
           Name nq = gen.fresh(s->id.s);

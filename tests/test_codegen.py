@@ -279,6 +279,24 @@ def test_tests_that_no_iteration_changes_move_out_of_the_state_loop(golden_dir):
     assert re.search(test, step(off)).start() > first_state(off)
 
 
+def test_values_picked_by_the_state_alone_are_computed_once(golden_dir):
+    """The stay transition's predecessor and score depend on the duration layer of the state, not on the step:
+    after the branches became selects they are hoisted into one register per state."""
+    import os
+    import oracle
+    hmm, seqs = oracle.reference_model_tables(os.path.join(golden_dir, "hmm_3mer_model.npz"), os.path.join(golden_dir, "hmm_signals.npz"))
+    n, S = seqs["num_instances"], hmm["num_states"]
+    a = np.zeros((n, S), dtype=np.float32)
+    args = [hmm, seqs, a, a.copy(), np.zeros(n, dtype=np.float32)]
+    par = {'inst': parpy.threads(n), 'state': parpy.threads(256)}
+    on = compiles(parpy.print_compiled(W.forward_kernel, args, opts_for(par)))
+    step = on[on.index("for (int t_"):]
+    assert re.search(r"int32_t inv_pick_\d+\[4\];", on) and re.search(r"float inv_pick_\d+\[4\];", on)
+    assert re.search(r"pred5_\d+ = inv_pick_\d+\[", step) and " ? " not in step[:step.index("__syncthreads")]
+    off = compiles(parpy.print_compiled(W.forward_kernel, args, opts_for(par, opt_if_convert=False)))
+    assert "inv_pick_" not in off
+
+
 def test_sddmm_kernels_compile():
     import oracle
     A, B, crows, cols, vals = W.make_sddmm(128, 16, 0.05)
