@@ -341,10 +341,13 @@ struct Pass {
           for (auto& kv : thn) assigned.insert(kv.first->name);
           for (auto& kv : els) assigned.insert(kv.first->name);
           bool independent = true;
-          auto reads_assigned = [&](const E& e) { visit_exprs(e, [&](const E& x) { if (x->k == Expr::Var && assigned.count(x->name)) independent = false; }); };
-          for (auto& kv : thn) reads_assigned(kv.second);
-          for (auto& kv : els) reads_assigned(kv.second);
-          reads_assigned(r->expr);
+          // (a value may read the variable it is assigned to -- its previous value, as in `w = c ? a : w` -- but no other)
+          auto reads_assigned = [&](const E& e, const Name* self) {
+            visit_exprs(e, [&](const E& x) { if (x->k == Expr::Var && assigned.count(x->name) && !(self && x->name == *self)) independent = false; });
+          };
+          for (auto& kv : thn) reads_assigned(kv.second, &kv.first->name);
+          for (auto& kv : els) reads_assigned(kv.second, &kv.first->name);
+          reads_assigned(r->expr, nullptr);
           if (independent && assigned.size() <= 4) {
             E test = r->expr;
             if (!cheap(test)) {   // reads memory: evaluated once, under a name (a cheap test is repeated, which lets a chain of elifs collapse)
@@ -360,7 +363,36 @@ struct Pass {
               if (!b) b = var;
               if (a->ty.sz != var->ty.sz) a = fold_expr(mk_convert(a, var->ty.sz));
               if (b->ty.sz != var->ty.sz) b = fold_expr(mk_convert(b, var->ty.sz));
-              out.push_back(mk_assign(var, mk_ifexpr(test, a, b, var->ty, r->i), r->i));
+              E picked = mk_ifexpr(test, a, b, var->ty, r->i);
+              // `x = init` a few statements up, nothing in between reading x or defining what the select reads:
+              // the select takes init's place there (`w = 0.5; if c: w = 2` -> `w = c ? 2 : 0.5`), which leaves a
+              // value that no longer depends on the variable's history
+              bool merged = false;
+              if (mentions(picked, name)) {
+                std::set<Name> between;
+                for (size_t back = out.size(); back-- > 0;) {
+                  const S& prev = out[back];
+                  bool def_like = (prev->k == Stmt::Def && prev->ty.is_scalar()) ||
+                                  (prev->k == Stmt::Assign && prev->dst->k == Expr::Var && prev->dst->ty.is_scalar());
+                  if (!def_like || !prev->expr || !cheap(prev->expr)) break;
+                  const Name& pn = prev->k == Stmt::Def ? prev->id : prev->dst->name;
+                  if (pn == name) {
+                    bool clash = false;
+                    visit_exprs(picked, [&](const E& x) { if (x->k == Expr::Var && between.count(x->name)) clash = true; });
+                    if (!clash && !mentions(prev->expr, name)) {
+                      std::map<Name, E> sub{{name, prev->expr}};
+                      auto np = clone(prev);
+                      np->expr = fold_expr(subst_vars(picked, sub));
+                      out[back] = np;
+                      merged = true;
+                    }
+                    break;
+                  }
+                  if (mentions(prev->expr, name)) break;
+                  between.insert(pn);
+                }
+              }
+              if (!merged) out.push_back(mk_assign(var, picked, r->i));
             }
             done = true;
           }
@@ -831,7 +863,6 @@ struct Pass {
             return re;
           };
           Stmts nbody = rewrite_stmts(*is.body, try_hoist);
-          if (hoisted.empty()) { out.push_back(s); continue; }
           // Arithmetic whose operands are all hoisted values (or literals) is invariant too: `trans1[..] +
           // trans2[..]` is computed once and takes one register per element instead of two.  Only values
           // with a single use are combined, so the register count never grows; same operations in the
@@ -925,7 +956,7 @@ struct Pass {
             };
             std::function<E(const E&)> pick = [&](const E& e) -> E {
               if (!e) return e;
-              if (e->k == Expr::IfExpr && e->ty.is_scalar() && elem_bytes(e->ty.sz) <= 4 && has_select(e)) {
+              if (e->k == Expr::IfExpr && e->ty.is_scalar() && has_select(e)) {
                 E v = fold_expr(subst_vars(e, defs));
                 bool pure = true;
                 visit_exprs(v, [&](const E& x) {
@@ -934,7 +965,7 @@ struct Pass {
                       x->k == Expr::Raw || x->k == Expr::AddrOf)
                     pure = false;
                 });
-                int64_t cost = is.slots;
+                int64_t cost = is.slots * std::max(1, elem_bytes(e->ty.sz) / 4);
                 if (pure && *budget >= cost) {
                   for (auto& h : hoisted)
                     if (h.load->k != Expr::Index && expr_eq(h.load, v)) {
@@ -968,6 +999,7 @@ struct Pass {
             };
             nbody = walk_picks(nbody);
           }
+          if (hoisted.empty()) { out.push_back(s); continue; }
           // loop nest that fills the registers, with the same thread mapping
           std::map<Name, Name> ren;
           Name nq = gen.fresh(s->id.s);

@@ -511,3 +511,45 @@ def test_branches_that_only_assign_scalars_keep_their_meaning_as_selects():
         got = np.zeros(N, dtype=np.float32)
         parpy.jit(pick_values)(x, y, got, N, opts=opts_for({'N': parpy.threads(N)}, opt_if_convert=flag))
         assert np.allclose(got, want, rtol=1e-6), flag
+
+
+def relax(x, y, N, M, T):
+    parpy.label('N')
+    for i in range(N):
+        for t in range(T):
+            parpy.label('M')
+            for j in range(M):
+                w = ops.float32(0.5)
+                k = j
+                if j % 3 == 0:
+                    w = ops.float32(2.0)
+                    k = (j + 5) % M
+                elif j % 3 == 1:
+                    w = ops.float32(-1.0)
+                y[i, j] = w * x[i, k] + ops.float32(t)
+            parpy.label('M')
+            for j in range(M):
+                x[i, j] = y[i, j] * ops.float32(0.5)
+
+
+def test_selects_on_the_iteration_alone_leave_the_time_loop():
+    N, M, T = 4, 256, 3
+    x = np.zeros((N, M), dtype=np.float32)
+    s = compiles(parpy.print_compiled(relax, [x, x.copy(), N, M, T], opts_for({'N': parpy.threads(N), 'M': parpy.threads(64)})))
+    body = s.split('extern "C" __global__')[1]
+    loop = body[body.index("for (int t_"):]
+    assert "inv_pick_" in body and " ? " not in loop[:loop.index("__syncthreads")]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("threads", [64, 100, 256])
+def test_selects_on_the_iteration_alone_keep_their_values(threads):
+    rng = np.random.default_rng(3)
+    N, M, T = 5, 300, 4
+    x0 = rng.uniform(-1, 1, (N, M)).astype(np.float32)
+    want_x, want_y = x0.copy(), np.zeros_like(x0)
+    relax(want_x, want_y, N, M, T)
+    for flags in ({}, {"opt_if_convert": False}, {"opt_hoist_invariant": False}):
+        got_x, got_y = x0.copy(), np.zeros_like(x0)
+        parpy.jit(relax)(got_x, got_y, N, M, T, opts=opts_for({'N': parpy.threads(N), 'M': parpy.threads(threads)}, **flags))
+        assert np.allclose(got_x, want_x, rtol=1e-5, atol=1e-6) and np.allclose(got_y, want_y, rtol=1e-5, atol=1e-6), flags
