@@ -231,6 +231,15 @@ def test_reference_model_with_state_vectors_larger_than_lds(threads):
     assert np.all(np.isfinite(want)) and np.allclose(got, want, atol=1e-4, rtol=1e-5), np.abs(got - want).max()
 
 
+@pytest.mark.parametrize("k,threads", [(1, 64), (2, 100), (3, 192), (3, 640), (4, 1024), (4, 2048)])
+def test_reference_format_models_with_random_tables(k, threads):
+    """Random tables in the reference model's layout, thread counts that do and do not divide the state count."""
+    hmm, seqs = _random_reference_model(k, n_reads=4, max_len=37, seed=100 * k + threads)
+    got = _run_reference_model(hmm, seqs, threads)
+    want = oracle.hmm_ref_forward(hmm, seqs, np.float32)
+    assert np.all(np.isfinite(want)) and np.allclose(got, want, atol=1e-4, rtol=1e-5), np.abs(got - want).max()
+
+
 def _run_synthetic(hmm, seqs, threads, **kw):
     hd, sd = W.to_device(hmm), W.to_device(seqs)
     n, S = seqs["num_instances"], hmm["num_states"]
