@@ -2003,7 +2003,8 @@ struct Coarsen {
           root->lo->k == Expr::Int && root->lo->iv == 0 && root->hi->k == Expr::Int))
       return false;
     const int64_t n = root->hi->iv, tpb = root->map.tpb;
-    if (n != root->map.n || tpb <= 0 || n % (4 * tpb) != 0 || n / 4 < 256 * 64) return false;
+    const int64_t launched = (n + WAVE_SIZE - 1) / WAVE_SIZE * WAVE_SIZE;
+    if (launched != root->map.n || tpb <= 0 || n / 4 < 256 * 64) return false;   // exactly one iteration per thread, and plenty
     if (k.grid.y != 1 || k.grid.z != 1 || k.block.y != 1 || k.block.z != 1) return false;
     bool straight = true;
     visit_stmts(root->body, [&](const S& c) {
@@ -2012,10 +2013,51 @@ struct Coarsen {
     if (!straight) return false;
     Pass probe(k, opts, gen);
     if (probe.vector_width(root) != 4) return false;   // 4-byte elements through parameters only
+    if (n % (4 * tpb) == 0) {
+      // whole workgroups of whole vectors: shrink the launch and let the vectorised remap do the rest
+      auto nr = clone(root);
+      nr->map.n = n / 4;
+      k.body = {S(nr)};
+      k.grid.x = n / 4 / tpb;
+      launch->grid = k.grid;
+      return true;
+    }
+    // any other n: thread q takes elements 4q .. 4q+3; the last thread may hold fewer and tests each of its own
+    ElemSize isz = opts.int_size();
+    Type ity = Type::scalar(isz);
+    const int64_t quads = (n + 3) / 4;
+    Name q = gen.fresh(root->id.s + "_q");
+    E qv = mk_var(q, ity);
+    auto elements = [&](bool guarded) {
+      Name u = gen.fresh(root->id.s + "_u");
+      E d = mk_binop(BinOp::Add, mk_binop(BinOp::Mul, qv, mk_int(4, isz), ity), mk_var(u, ity), ity);
+      Stmts ib;
+      ib.push_back(mk_def(root->id, ity, d, root->i));
+      for (auto& b : root->body) ib.push_back(b);
+      if (guarded) {
+        Stmts inner = {ib.begin() + 1, ib.end()};
+        ib = {ib[0], mk_if(mk_binop(BinOp::Lt, mk_var(root->id, ity), mk_int(n, isz), Type::scalar(ElemSize::Bool)), inner, {})};
+      }
+      auto loop = std::const_pointer_cast<Stmt>(std::static_pointer_cast<const Stmt>(
+          mk_for(u, mk_int(0, isz), mk_int(4, isz), 1, ib, LoopPar(), root->i)));
+      loop->unroll = true;
+      return S(loop);
+    };
+    Stmts body;
+    if (n % 4 == 0) {
+      body = {elements(false)};
+    } else {
+      E whole = mk_binop(BinOp::Leq, mk_binop(BinOp::Add, mk_binop(BinOp::Mul, qv, mk_int(4, isz), ity), mk_int(4, isz), ity), mk_int(n, isz),
+                         Type::scalar(ElemSize::Bool));
+      body = {mk_if(whole, {elements(false)}, {elements(true)})};
+    }
     auto nr = clone(root);
-    nr->map.n = n / 4;
+    nr->id = q;
+    nr->hi = mk_int(quads, isz);
+    nr->body = body;
+    nr->map.n = (quads + WAVE_SIZE - 1) / WAVE_SIZE * WAVE_SIZE;
     k.body = {S(nr)};
-    k.grid.x = n / 4 / tpb;
+    k.grid.x = (nr->map.n + tpb - 1) / tpb;
     launch->grid = k.grid;
     return true;
   }

@@ -142,6 +142,12 @@ def test_one_element_per_thread_becomes_four_on_large_element_wise_launches():
     x = np.zeros(n, dtype=np.float32)
     s = compiles(parpy.print_compiled(K.axpy, [2.0, x, x, x.copy(), n], opts_for({'N': parpy.threads(n)})))
     assert launch(s) == [(str(n // 4 // 1024), "1", "1", "1024", "1", "1")] and re.search(r"_u_\d+ < 4;", s)
+    # any other length: thread q takes 4q .. 4q+3 and only the last thread tests its elements one by one
+    r = 1_000_003
+    xr = np.zeros(r, dtype=np.float32)
+    s = compiles(parpy.print_compiled(K.axpy, [2.0, xr, xr, xr.copy(), r], opts_for({'N': parpy.threads(r)})))
+    assert launch(s) == [(str((250_001 + 1023) // 1024), "1", "1", "1024", "1", "1")]
+    assert "< 250001)" in s and "+ 4) <= 1000003)" in s and "< 1000003)" in s
     # a launch that would leave CUs short of threads keeps one element per thread; so does an unaligned argument
     m = 1 << 15
     s = compiles(parpy.print_compiled(K.axpy, [2.0, x[:m], x[:m], x[:m].copy(), m], opts_for({'N': parpy.threads(m)})))

@@ -588,6 +588,19 @@ def test_two_host_threads_share_one_compiled_function():
         assert torch.allclose(outs[i], xs[i].sum(dim=1), rtol=1e-12, atol=1e-12)
 
 
+@pytest.mark.parametrize("n", [1 << 20, 1_000_003, 100_001, 65_538, 40_000])
+def test_element_wise_launch_with_one_element_per_thread(n):
+    """`parpy.threads(n)` on n elements: large launches run four elements per thread, whatever n is; the tail is exact."""
+    rng = np.random.default_rng(n)
+    x, y = rng.standard_normal(n).astype(np.float32), rng.standard_normal(n).astype(np.float32)
+    xd, yd = torch.from_numpy(x).cuda(), torch.from_numpy(y).cuda()
+    out = torch.full((n + 8,), 7.0, dtype=torch.float32, device="cuda")      # room behind the end to catch stray stores
+    parpy.jit(K.axpy)(2.0, xd, yd, out[:n], n, opts=opts_for({'N': parpy.threads(n)}))
+    want = (2.0 * x.astype(np.float64) + y.astype(np.float64)).astype(np.float32)
+    got = out.cpu().numpy()
+    assert np.array_equal(got[:n], want) and np.all(got[n:] == 7.0)
+
+
 def test_random_shapes_and_thread_counts():
     """Row reductions, softmax and the element-wise copy over seeded random shapes and thread counts:
     extents that do and do not divide by the vector width, the wavefront and the block size."""
