@@ -190,8 +190,16 @@ def test_forward_written_with_value_returning_helpers(golden_dir, threads):
 def test_forward_3mer_golden_unoptimised(golden_dir):
     hmm, seqs, exp = _golden(golden_dir, 3)
     got = _run_reference_model(hmm, seqs, 512, opt_lds_rows=False, opt_vectorize=False, opt_hoist_invariant=False,
-                               opt_narrow_index=False)
+                               opt_narrow_index=False, opt_unswitch_uniform=False, opt_offset32=False, opt_if_convert=False,
+                               opt_drop_barriers=False, opt_reg_cache=False, opt_lane_split=False, opt_nontemporal=False)
     assert np.allclose(got, exp, atol=1e-5, rtol=1e-5), np.abs(got - exp).max()
+
+
+@pytest.mark.parametrize("flag", ["opt_unswitch_uniform", "opt_offset32", "opt_if_convert", "opt_hoist_invariant", "opt_lds_rows", "opt_vectorize"])
+def test_forward_3mer_golden_with_one_pass_off(golden_dir, flag):
+    hmm, seqs, exp = _golden(golden_dir, 3)
+    got = _run_reference_model(hmm, seqs, 1024, **{flag: False})
+    assert np.allclose(got, exp, atol=1e-5, rtol=1e-5), (flag, np.abs(got - exp).max())
 
 
 def test_forward_5mer_golden(golden_dir):
