@@ -101,6 +101,27 @@ int64_t parpy_hip_plan_launch_count(void* plan);
 
 int32_t parpy_hip_plan_destroy(void* plan);
 
+/* ---- a run that allocates nothing ---- */
+
+/* No counterpart in the reference (its generated entry points call
+ * cudaMallocAsync for every temporary, src/cuda/codegen.rs:179-202).  For
+ * callers that cannot allocate device memory: tight serving loops, code under
+ * a HIP graph capture elsewhere in the process, harnesses that forbid
+ * hipMalloc.  Same arguments, result and status as parpy_hip_plan_run, but the
+ * plan's device temporaries (partial results of multi-block reductions, locals
+ * that cross kernels, transposed operands) are carved out of one array of
+ * PARPY_HIP_SCRATCH_BYTES that is part of the library's code object, and no
+ * hipMalloc / hipFree or other allocating call is made.  A plan whose
+ * temporaries need more fails with a message and runs nothing.  Launches are
+ * eager on the null stream (graph replay and kept temporaries do not apply).
+ * Every call on a GPU uses that GPU's one array and temporaries start with
+ * whatever the previous call left there (the kernels write a temporary before
+ * they read it, as with a fresh allocation); two calls that overlap on one
+ * GPU -- from two host threads, or on work still in flight on another stream
+ * -- race on it. */
+#define PARPY_HIP_SCRATCH_BYTES (16u << 20)
+int32_t parpy_hip_plan_run_noalloc(void* plan, void* const* args, int32_t nargs);
+
 #ifdef __cplusplus
 }
 #endif

@@ -160,8 +160,16 @@ def get_wrapper(name, key, plan_text, opts):
         if lib.parpy_hip_plan_run(plan, arr, len(ptrs)) != 0:
             raise RuntimeError(f"{lib.parpy_get_error_message().decode('ascii', 'replace')}")
 
+    def run_noalloc(ptrs):
+        """As `run_pointers`, through the entry point that allocates nothing: the plan's temporaries
+        come out of the runtime library's fixed scratch array (parpy_hip_plan_run_noalloc)."""
+        arr = (ctypes.c_void_p * max(1, len(ptrs)))(*ptrs)
+        if lib.parpy_hip_plan_run_noalloc(plan, arr, len(ptrs)) != 0:
+            raise RuntimeError(f"{lib.parpy_get_error_message().decode('ascii', 'replace')}")
+
     wrapper.__name__ = name
     wrapper.run_pointers = run_pointers
+    wrapper.run_noalloc = run_noalloc
     wrapper.timed = timed
     wrapper.plan = plan
     wrapper.launch_count = lambda: lib.parpy_hip_plan_launch_count(plan)

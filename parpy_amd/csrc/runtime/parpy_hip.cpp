@@ -91,6 +91,34 @@ struct HStmt {
 
 constexpr int64_t KEEP_LIMIT = int64_t(1) << 30;
 
+}  // namespace
+
+// Device memory for the temporaries of parpy_hip_plan_run_noalloc: part of the library's code
+// object, so every GPU the library runs on holds one copy from the first use until the process
+// ends.  The name below is only a host-side handle; the device address is looked up once per
+// device with hipGetSymbolAddress and that address is what plans receive.
+static __device__ __align__(256) unsigned char scratch[PARPY_HIP_SCRATCH_BYTES];
+
+namespace {
+
+constexpr int MAX_DEVICES = 64;
+std::mutex g_scratch_mu;
+unsigned char* g_scratch_ptr[MAX_DEVICES] = {};
+
+// Device address of the scratch array on the current device (nullptr + message on failure).
+unsigned char* scratch_on_current_device() {
+  int dev = -1;
+  if (check(hipGetDevice(&dev), "hipGetDevice")) return nullptr;
+  if (dev < 0 || dev >= MAX_DEVICES) { fail("device ordinal out of range for the scratch table"); return nullptr; }
+  std::lock_guard<std::mutex> g(g_scratch_mu);
+  if (!g_scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    if (check(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)")) return nullptr;
+    g_scratch_ptr[dev] = (unsigned char*)ptr;
+  }
+  return g_scratch_ptr[dev];
+}
+
 struct Plan {
   hipModule_t module = nullptr;
   std::vector<hipFunction_t> fns;
@@ -124,6 +152,12 @@ struct Plan {
   // foreign-function calls that release the interpreter lock: two threads calling one compiled
   // function must take turns (the device work they enqueue is ordered by the stream anyway).
   std::mutex mu;
+  // Set for the duration of a run through parpy_hip_plan_run_noalloc: temporaries are carved out of
+  // the scratch array (stack discipline) instead of being allocated.
+  unsigned char* scratch_base = nullptr;
+  int64_t scratch_top = 0;
+  struct Carved { int slot; int64_t off; };
+  std::vector<Carved> carved;
 };
 
 struct PlanBuilder {
@@ -397,6 +431,18 @@ int32_t run_stmt(Plan& p, const HStmt& s) {
       p.env[s.slot] = eval(p, s.a);
       return 0;
     case HStmt::Alloc: {
+      if (p.scratch_base) {
+        int64_t off = (p.scratch_top + 255) & ~int64_t(255);
+        if (s.nbytes < 0 || off + s.nbytes > (int64_t)PARPY_HIP_SCRATCH_BYTES)
+          return fail("the device temporaries of this plan need " + std::to_string(off + s.nbytes) +
+                      " bytes, more than the " + std::to_string((int64_t)PARPY_HIP_SCRATCH_BYTES) +
+                      " bytes of scratch memory that parpy_hip_plan_run_noalloc has; use parpy_hip_plan_run");
+        p.carved.push_back({s.slot, off});
+        p.scratch_top = off + s.nbytes;
+        p.env[s.slot].t = Val::P;
+        p.env[s.slot].p = p.scratch_base + off;
+        return 0;
+      }
       if (p.kept.size() < p.env.size()) p.kept.resize(p.env.size());
       Plan::Kept& kp = p.kept[s.slot];
       if (kp.ptr && kp.nbytes == s.nbytes && !kp.in_use) {
@@ -424,6 +470,15 @@ int32_t run_stmt(Plan& p, const HStmt& s) {
       return 0;
     }
     case HStmt::Free: {
+      if (p.scratch_base) {
+        // the most recent temporary gives its space back; others stay carved until the run ends
+        if (!p.carved.empty() && p.carved.back().slot == s.slot) {
+          p.scratch_top = p.carved.back().off;
+          p.carved.pop_back();
+        }
+        p.env[s.slot].p = nullptr;
+        return 0;
+      }
       void* ptr = p.env[s.slot].p;
       p.env[s.slot].p = nullptr;
       if ((size_t)s.slot < p.kept.size() && p.kept[s.slot].ptr == ptr && ptr) {
@@ -451,7 +506,12 @@ int32_t run_stmts(Plan& p, const std::vector<HStmt>& ss) {
 
 extern "C" {
 
-void parpy_init(int64_t) {}
+void parpy_init(int64_t) {
+  // look up this device's scratch array now when a device is there; a later call retries
+  int n = 0;
+  if (hipGetDeviceCount(&n) != hipSuccess || n == 0) { (void)hipGetLastError(); return; }
+  if (!scratch_on_current_device()) g_error = "no error";
+}
 
 int32_t parpy_sync(void) { return check(hipDeviceSynchronize(), "hipDeviceSynchronize"); }
 
@@ -693,6 +753,27 @@ int32_t parpy_hip_plan_run_timed(void* plan, void* const* args, int32_t nargs, f
   if (int32_t rc = check(hipEventRecord(p.ev_stop, nullptr), "hipEventRecord")) return rc;
   if (int32_t rc = check(hipEventSynchronize(p.ev_stop), "hipEventSynchronize")) return rc;
   return check(hipEventElapsedTime(elapsed_ms, p.ev_start, p.ev_stop), "hipEventElapsedTime");
+}
+
+int32_t parpy_hip_plan_run_noalloc(void* plan, void* const* args, int32_t nargs) {
+  Plan& p = *(Plan*)plan;
+  std::lock_guard<std::mutex> turn(p.mu);
+  unsigned char* base = scratch_on_current_device();
+  if (!base) return 1;
+  if (nargs != p.nparams)
+    return fail("launch plan expects " + std::to_string(p.nparams) + " pointer arguments, received " + std::to_string(nargs));
+  if (!p.module) return fail("launch plan was created without a loaded module");
+  for (int k = 0; k < nargs; ++k) {
+    p.env[k].t = Val::P;
+    p.env[k].p = args[k];
+  }
+  p.scratch_base = base;
+  p.scratch_top = 0;
+  p.carved.clear();
+  p.launches = 0;
+  int32_t rc = run_stmts(p, p.body);   // eager launches on the null stream; no graph, no kept temporaries
+  p.scratch_base = nullptr;
+  return rc;
 }
 
 int64_t parpy_hip_plan_launch_count(void* plan) { return ((Plan*)plan)->launches; }

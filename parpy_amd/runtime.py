@@ -15,7 +15,7 @@ from .options import CompileBackend
 
 PARPY_NATIVE_PATH = pathlib.Path(__file__).parent / "csrc" / "runtime"
 PARPY_HIP_BASE_LIB_PATH = pathlib.Path(__file__).parent / "libparpy_hip.so"
-HIPCC_FLAGS = ["-O2", "-fPIC", "-shared", "-std=c++17",
+HIPCC_FLAGS = ["-O2", "-fPIC", "-shared", "-std=c++17", "--offload-arch=gfx950",
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
 libs = {}
@@ -69,6 +69,8 @@ def init_library(libpath):
     lib.parpy_hip_plan_run.restype = i32
     lib.parpy_hip_plan_run_timed.argtypes = [vp, ctypes.POINTER(vp), i32, ctypes.POINTER(ctypes.c_float)]
     lib.parpy_hip_plan_run_timed.restype = i32
+    lib.parpy_hip_plan_run_noalloc.argtypes = [vp, ctypes.POINTER(vp), i32]
+    lib.parpy_hip_plan_run_noalloc.restype = i32
     lib.parpy_hip_plan_set_graph.argtypes = [vp, i32]
     lib.parpy_hip_plan_set_graph.restype = i32
     lib.parpy_hip_plan_graph_replays.argtypes = [vp]
