@@ -327,6 +327,9 @@ Interval range_impl(const E& e, const RangeEnv& env) {
     }
     case Expr::BinOpE: {
       Interval a = expr_range(e->args[0], env), b = expr_range(e->args[1], env);
+      // the smaller of two values is bounded above by either one alone (a loop that runs to min(n, len[i]))
+      if (e->bop == BinOp::Min && a.known != b.known) return iv(INT64_MIN, a.known ? a.hi : b.hi);
+      if (e->bop == BinOp::Max && a.known != b.known) return iv(a.known ? a.lo : b.lo, INT64_MAX);
       if (!a.known || !b.known) return none;
       int64_t r0, r1, r2, r3;
       switch (e->bop) {

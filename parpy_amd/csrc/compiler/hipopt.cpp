@@ -232,6 +232,190 @@ struct Pass {
     }
   };
 
+  // ================================================================ short counted loops inside one iteration
+  // `for u in range(4): ...` written inside the body of a parallel loop (the four states of a group, the
+  // taps of a small stencil) is expanded in place: one copy of the body per value of u, with the copy's
+  // local variables renamed and u replaced by its value.  Every index then depends on the thread's own
+  // iteration alone, which is the form the invariant-load and register passes below work on, and the tests
+  // on u fold away.  Only loops of at most 8 iterations whose body is straight-line code and value-picking
+  // branches are expanded.
+  static bool straight_line(const Stmts& ss) {
+    for (auto& s : ss) {
+      if (s->k == Stmt::If) { if (!straight_line(s->body) || !straight_line(s->els)) return false; continue; }
+      if (s->k != Stmt::Def && s->k != Stmt::Assign) return false;
+    }
+    return true;
+  }
+
+  Stmts expand_short_loops(const Stmts& ss, bool in_par) {
+    Stmts out;
+    for (auto& s : ss) {
+      int64_t n = s->k == Stmt::For && s->map.k == GpuMap::None ? const_extent(s) : -1;
+      if (in_par && n >= 1 && n <= 8 && straight_line(s->body)) {
+        std::vector<Name> locals;
+        visit_stmts(s->body, [&](const S& c) { if (c->k == Stmt::Def) locals.push_back(c->id); });
+        for (int64_t it = 0; it < n; ++it) {
+          std::map<Name, E> sub;
+          std::map<Name, Name> ren;
+          sub[s->id] = mk_int(s->lo->iv + it * s->step, isz);
+          for (auto& l : locals) ren[l] = gen.fresh(l.s);
+          std::function<Stmts(const Stmts&)> copy = [&](const Stmts& b) {
+            Stmts o;
+            for (auto& c : b) {
+              auto r = clone(c);
+              auto fix = [&](const E& e) {
+                return rewrite_expr(e, [&](const E& x) -> E {
+                  if (x->k != Expr::Var) return x;
+                  auto si = sub.find(x->name);
+                  if (si != sub.end()) return si->second;
+                  auto ri = ren.find(x->name);
+                  if (ri == ren.end()) return x;
+                  auto v = std::make_shared<Expr>(*x);
+                  v->name = ri->second;
+                  return E(v);
+                });
+              };
+              if (r->dst) r->dst = fix(r->dst);
+              if (r->expr) r->expr = fix(r->expr);
+              if (r->k == Stmt::Def) r->id = ren[c->id];
+              r->body = copy(c->body);
+              r->els = copy(c->els);
+              o.push_back(r);
+            }
+            return o;
+          };
+          for (auto& c : fold_stmts(copy(s->body))) out.push_back(c);
+        }
+        continue;
+      }
+      auto r = clone(s);
+      bool par = in_par || (s->k == Stmt::For && s->map.k != GpuMap::None);
+      r->body = expand_short_loops(s->body, par);
+      r->els = expand_short_loops(s->els, par);
+      out.push_back(r);
+    }
+    return out;
+  }
+
+  // ================================================================ guards that only ever switch off
+  // `for t in range(lo, hi): ... if t < X: <work>` where X does not change while the loop runs, every
+  // effect of the body sits under that test and X is the same for all threads of the workgroup: once
+  // t reaches X no later iteration does anything, so the loop runs to min(hi, X) and the test goes.
+  // The HMM kernels walk every read to the length of the longest one this way; with the bound in the
+  // loop a workgroup ends with its read (its compute unit is free for the next one) and the step no
+  // longer carries the test through every state.
+  static E strip_converts(const E& e) { return e->k == Expr::Convert ? strip_converts(e->args[0]) : e; }
+
+  Stmts guards_to_bounds(const Stmts& ss) {
+    std::set<Name> params = param_names();
+    std::set<Name> written = written_arrays();
+    Stmts out;
+    for (auto& s : ss) {
+      bool seq = s->k == Stmt::For && s->map.k == GpuMap::None && !s->unroll && s->step == 1;
+      E bound;
+      bool ok = seq;
+      std::set<Name> local;
+      if (seq) {
+        local.insert(s->id);
+        visit_stmts(s->body, [&](const S& c) {
+          if (c->k == Stmt::Def || c->k == Stmt::For) local.insert(c->id);
+          if (c->k == Stmt::Assign && c->dst->k == Expr::Var) local.insert(c->dst->name);
+        });
+      }
+      auto guard_of = [&](const S& c, E* x) {
+        if (c->k != Stmt::If || !c->els.empty() || c->expr->k != Expr::BinOpE) return false;
+        const E &a = c->expr->args[0], &b = c->expr->args[1];
+        E t, other;
+        if (c->expr->bop == BinOp::Lt) { t = a; other = b; }
+        else if (c->expr->bop == BinOp::Gt) { t = b; other = a; }
+        else return false;
+        E tv = strip_converts(t);
+        if (tv->k != Expr::Var || tv->name != s->id) return false;
+        bool uniform = true;
+        visit_exprs(other, [&](const E& y) {
+          if (y->k == Expr::Var && local.count(y->name)) uniform = false;
+          if (y->k == Expr::Index && !(y->args[0]->k == Expr::Var && params.count(y->args[0]->name) && !written.count(y->args[0]->name)))
+            uniform = false;
+          if (y->k == Expr::Call || y->k == Expr::Raw || y->k == Expr::RegElem || y->k == Expr::ThreadIdx || y->k == Expr::AddrOf) uniform = false;
+        });
+        if (!uniform || !other->ty.is_scalar() || !is_int(other->ty.sz)) return false;
+        *x = other;
+        return true;
+      };
+      // statements without effects outside the iteration: definitions and assignments of the iteration's own scalars
+      std::function<bool(const Stmts&)> effect_free = [&](const Stmts& b) {
+        for (auto& c : b) {
+          if (c->k == Stmt::Def) continue;
+          if (c->k == Stmt::Assign && c->dst->k == Expr::Var) continue;
+          if (c->k == Stmt::If && effect_free(c->body) && effect_free(c->els)) continue;
+          return false;
+        }
+        return true;
+      };
+      int guards = 0;
+      std::function<Stmts(const Stmts&)> strip = [&](const Stmts& b) -> Stmts {
+        Stmts o;
+        for (auto& c : b) {
+          E x;
+          if (guard_of(c, &x)) {
+            if (bound && !expr_eq(bound, x)) { ok = false; return o; }
+            bound = x;
+            ++guards;
+            for (auto& g : c->body) o.push_back(g);
+            continue;
+          }
+          if (c->k == Stmt::Sync || c->k == Stmt::SyncPoint) { o.push_back(c); continue; }
+          if (c->k == Stmt::For && c->map.k != GpuMap::None) {
+            auto r = clone(c);
+            r->body = strip(c->body);
+            o.push_back(r);
+            continue;
+          }
+          if (effect_free({c})) { o.push_back(c); continue; }
+          ok = false;
+          return o;
+        }
+        return o;
+      };
+      if (seq) {
+        // an assignment outside the tests to a variable that lives beyond the loop would see fewer iterations
+        std::set<Name> defined_inside;
+        visit_stmts(s->body, [&](const S& c) { if (c->k == Stmt::Def || c->k == Stmt::For) defined_inside.insert(c->id); });
+        Stmts body = strip(s->body);
+        std::function<void(const Stmts&, bool)> check = [&](const Stmts& b, bool) {};
+        if (ok && guards > 0) {
+          bool escapes = false;
+          std::function<void(const Stmts&)> scan = [&](const Stmts& b) {
+            for (auto& c : b) {
+              E x;
+              if (guard_of(c, &x)) continue;   // what a test covers ran in the same iterations before
+              if (c->k == Stmt::Assign && c->dst->k == Expr::Var && !defined_inside.count(c->dst->name)) escapes = true;
+              scan(c->body);
+              scan(c->els);
+            }
+          };
+          scan(s->body);
+          if (!escapes) {
+            auto r = clone(s);
+            E x = bound->ty.sz == s->hi->ty.sz ? bound : mk_convert(bound, s->hi->ty.sz);
+            // evaluated once, in front of the loop: a load in the loop test would be repeated behind every barrier
+            Name end = gen.fresh(s->id.s + "_end");
+            out.push_back(mk_def(end, s->hi->ty, mk_binop(BinOp::Min, s->hi, x, s->hi->ty, s->i), s->i));
+            r->hi = mk_var(end, s->hi->ty);
+            r->body = guards_to_bounds(body);
+            out.push_back(r);
+            continue;
+          }
+        }
+      }
+      auto r = clone(s);
+      r->body = guards_to_bounds(s->body);
+      r->els = guards_to_bounds(s->els);
+      out.push_back(r);
+    }
+    return out;
+  }
+
   // ================================================================ conditions no iteration changes
   // A parallel loop whose whole body is `if (c) A else B`, with c the same for every iteration (it
   // mentions neither the loop variable nor anything the body defines or assigns, and loads only from
@@ -665,13 +849,18 @@ struct Pass {
   // with the rewrite, 60 us without.)  Pointers into LDS have no such cost.
   int vector_width(const S& loop) {
     int v = 0;
-    bool through_global_alias = false;
+    bool through_global_alias = false, owns_runs = false;
     std::set<Name> params = param_names();
     std::function<void(const E&)> scan = [&](const E& e) {
       visit_exprs(e, [&](const E& x) {
         if (x->k != Expr::Index) return;
         E rest;
-        if (!affine_unit(x->args[1], loop->id, &rest)) return;
+        if (!affine_unit(x->args[1], loop->id, &rest)) {
+          // an iteration that already owns a run of 16 bytes or more (`a[4*d + c]`): neighbouring lanes sit on
+          // neighbouring runs, and giving a thread V consecutive iterations would put them V runs apart
+          if (strided_run(x->args[1], loop->id) * elem_bytes(x->ty.sz) >= 16) owns_runs = true;
+          return;
+        }
         const E& base = x->args[0];
         if (base->k == Expr::Var && !params.count(base->name) && base->ty.mem != Mem::LDS) through_global_alias = true;
         // (the same holds for every global array when the call passed one that is not 16-byte aligned)
@@ -682,7 +871,23 @@ struct Pass {
       });
     };
     visit_stmts(loop->body, [&](const S& s) { scan(s->dst); scan(s->expr); scan(s->lo); scan(s->hi); });
-    return through_global_alias ? 0 : v;
+    return through_global_alias || owns_runs ? 0 : v;
+  }
+
+  // c when idx == c * d + rest with rest free of d and c a constant > 1, else 0
+  static int64_t strided_run(const E& idx, const Name& d) {
+    if (idx->k != Expr::BinOpE) return 0;
+    const E &a = idx->args[0], &b = idx->args[1];
+    if (idx->bop == BinOp::Mul) {
+      if (a->k == Expr::Int && b->k == Expr::Var && b->name == d) return a->iv > 1 ? a->iv : 0;
+      if (b->k == Expr::Int && a->k == Expr::Var && a->name == d) return b->iv > 1 ? b->iv : 0;
+      return 0;
+    }
+    if (idx->bop == BinOp::Add || idx->bop == BinOp::Sub) {
+      if (!mentions(b, d)) return strided_run(a, d);
+      if (idx->bop == BinOp::Add && !mentions(a, d)) return strided_run(b, d);
+    }
+    return 0;
   }
 
   Stmts vectorize(const Stmts& ss) {
@@ -2088,6 +2293,8 @@ void hip_optimize(Program& p, const Options& opts, NameGen& gen) {
     Pass pass(k, opts, gen);
     if (opts.opt_unswitch) pass.unswitch_aliases();
     if (opts.opt_mfma_sddmm) k.body = pass.mfma_dot(k.body);
+    if (opts.opt_expand_short_loops) k.body = pass.expand_short_loops(k.body, false);
+    if (opts.opt_guard_bounds) k.body = pass.guards_to_bounds(k.body);
     if (opts.opt_unswitch_uniform) k.body = pass.hoist_uniform_conditions(k.body);
     if (opts.opt_if_convert) k.body = pass.if_convert(k.body);
     if (opts.opt_lds_rows) pass.lds_rows();

@@ -120,6 +120,19 @@ struct parpy_op_min {
 };
 template <class T> __device__ __forceinline__ T parpy_max(T a, T b) { return parpy_op_max()(a, b); }
 template <class T> __device__ __forceinline__ T parpy_min(T a, T b) { return parpy_op_min()(a, b); }
+// fp32 max / min of a statement as the one machine instruction (three operands: v_max3 / v_min3).  Through
+// fmaxf() every operand that comes from memory is first passed through a quieting `v_max_f32 x, x`, because a
+// signalling NaN must not reach the instruction under the C rules.  The instruction returns the other operand
+// when one is a quiet NaN -- the behaviour that log-space kernels rely on -- and no arithmetic produces a
+// signalling NaN.  The `c` forms take a compile-time constant as last operand (kept in a scalar register).
+__device__ __forceinline__ float parpy_fmax(float a, float b) { float r; asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b)); return r; }
+__device__ __forceinline__ float parpy_fmin(float a, float b) { float r; asm("v_min_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b)); return r; }
+__device__ __forceinline__ float parpy_fmaxc(float a, float c) { float r; asm("v_max_f32 %0, %1, %2" : "=v"(r) : "s"(c), "v"(a)); return r; }
+__device__ __forceinline__ float parpy_fminc(float a, float c) { float r; asm("v_min_f32 %0, %1, %2" : "=v"(r) : "s"(c), "v"(a)); return r; }
+__device__ __forceinline__ float parpy_fmax3(float a, float b, float c) { float r; asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c)); return r; }
+__device__ __forceinline__ float parpy_fmin3(float a, float b, float c) { float r; asm("v_min3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c)); return r; }
+__device__ __forceinline__ float parpy_fmax3c(float a, float b, float c) { float r; asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "s"(c)); return r; }
+__device__ __forceinline__ float parpy_fmin3c(float a, float b, float c) { float r; asm("v_min3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "s"(c)); return r; }
 // reduce over each row of 16 lanes; afterwards every lane of a row holds the row's result
 template <class Op, class T> __device__ __forceinline__ T parpy_row_reduce(T v) {
   Op op;
@@ -314,6 +327,22 @@ struct DevicePrinter {
     return std::string(base) + "f";
   }
 
+  // fp32 values that come straight from memory (a load, or a variable that only names one): what the compiler
+  // would have to quiet before a max / min; maxima and minima of such values count as well, since they are
+  // printed as opaque instructions
+  std::set<Name> loaded_f32;
+  static bool float_literal(const E& x) {
+    return x->k == Expr::Float || (x->k == Expr::UnOpE && x->uop == UnOp::Sub && x->args[0]->k == Expr::Float) ||
+           (x->k == Expr::Convert && float_literal(x->args[0]));
+  }
+  bool straight_from_memory(const E& x) const {
+    if (x->k == Expr::Index || x->k == Expr::RegElem) return true;
+    if (x->k == Expr::Var) return loaded_f32.count(x->name) > 0;
+    if (x->k == Expr::BinOpE && (x->bop == BinOp::Max || x->bop == BinOp::Min) && x->args[0]->ty.sz == ElemSize::F32)
+      return straight_from_memory(x->args[0]) || straight_from_memory(x->args[1]);
+    return false;
+  }
+
   std::string pexpr(const E& e) {
     if (is_i64(e)) return pint(e).s;
     return pexpr_plain(e);
@@ -375,6 +404,22 @@ struct DevicePrinter {
         switch (e->bop) {
           case BinOp::Max: case BinOp::Min: {
             const char* base = e->bop == BinOp::Max ? "max" : "min";
+            if (sz == ElemSize::F32 && straight_from_memory(e)) {
+              // one v_max / v_min, or v_max3 / v_min3 for a nested pair (see the preamble for why not fmaxf)
+              auto same = [&](const E& x) { return x->k == Expr::BinOpE && x->bop == e->bop && x->args[0]->ty.sz == ElemSize::F32; };
+              std::string f = std::string("parpy_f") + base;
+              if (float_literal(e->args[1])) {
+                if (same(e->args[0]) && !float_literal(e->args[0]->args[0]) && !float_literal(e->args[0]->args[1]))
+                  return f + "3c(" + pexpr(e->args[0]->args[0]) + ", " + pexpr(e->args[0]->args[1]) + ", " + b + ")";
+                return f + "c(" + a + ", " + b + ")";
+              }
+              if (float_literal(e->args[0])) return f + "c(" + b + ", " + a + ")";
+              if (same(e->args[0]) && !float_literal(e->args[0]->args[0]) && !float_literal(e->args[0]->args[1]))
+                return f + "3(" + pexpr(e->args[0]->args[0]) + ", " + pexpr(e->args[0]->args[1]) + ", " + b + ")";
+              if (same(e->args[1]) && !float_literal(e->args[1]->args[0]) && !float_literal(e->args[1]->args[1]))
+                return f + "3(" + a + ", " + pexpr(e->args[1]->args[0]) + ", " + pexpr(e->args[1]->args[1]) + ")";
+              return f + "(" + a + ", " + b + ")";
+            }
             if (sz == ElemSize::F32) return std::string("f") + base + "f(" + a + ", " + b + ")";
             if (sz == ElemSize::F64) return std::string("f") + base + "(" + a + ", " + b + ")";
             if (sz == ElemSize::F16) return std::string("((_Float16)f") + base + "f((float)" + paren(a) + ", (float)" + paren(b) + "))";
@@ -623,6 +668,7 @@ struct DevicePrinter {
         bool is64 = s->ty.is_scalar() && s->ty.sz == ElemSize::I64;
         bool fixed = !reassigned.count(s->id);
         if (fixed && r.known) ranges[s->id] = r;
+        if (fixed && s->ty.is_scalar() && s->ty.sz == ElemSize::F32 && s->expr && straight_from_memory(s->expr)) loaded_f32.insert(s->id);
         bool narrow = opts.opt_narrow_index && is64 && fixed && fits32(r);
         if (narrow) narrow_vars.insert(s->id);
         std::string rhs = pexpr(s->expr);

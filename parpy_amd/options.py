@@ -254,6 +254,8 @@ class CompileOptions:
         'opt_offset32': None,
         'opt_if_convert': None,
         'opt_noalias_scopes': None,
+        'opt_expand_short_loops': None,
+        'opt_guard_bounds': None,
         'reg_budget': None,   # registers per thread the caching passes may claim (None: by block size)
         'assume_aligned': None,   # set by the driver: False when an array argument is not 16-byte aligned
     }

@@ -239,6 +239,106 @@ def forward_syn(hmm, seqs, result, alpha1, alpha2):
         forward_syn_lse(hmm, seqs, result, alpha1, alpha2, inst)
 
 
+# ---------------------------------------------------------------- HMM forward, synthetic model, four states at a time
+@parpy.jit
+def syn4_state(e1, e2, e3, e4, t1, t2, t3, t4, w, own, m, emission):
+    """New score of one state of a group whose scores do not exceed the predecessors' by more than e^80."""
+    return m + log(e1 * t1 + e2 * t2 + e3 * t3 + e4 * t4 + w * exp(own - m)) + emission
+
+
+@parpy.jit
+def syn4_state_wide(e1, e2, e3, e4, t1, t2, t3, t4, w, own, m, emission):
+    """The same for any scores: the sum is referred to the larger of `own` and `m`, so that the one exponential
+    taken here never exceeds one."""
+    s = e1 * t1 + e2 * t2 + e3 * t3 + e4 * t4
+    e = exp(-abs(own - m))
+    total = s + w * e
+    base = m
+    if own > m:
+        total = w + s * e
+        base = own
+    return base + log(total) + emission
+
+
+@parpy.jit
+def forward_syn4_step(hmm, seqs, alpha1, alpha2, inst, t):
+    alpha_src = alpha2
+    alpha_dst = alpha1
+    if t & 1:
+        alpha_src = alpha1
+        alpha_dst = alpha2
+    o = seqs["data"][inst, t]
+    parpy.label('state')
+    for q in range(hmm["num_states"] // 4):
+        if t < seqs["lens"][inst]:
+            nq = hmm["num_states"] // 4
+            a1 = alpha_src[inst, q]
+            a2 = alpha_src[inst, nq + q]
+            a3 = alpha_src[inst, 2 * nq + q]
+            a4 = alpha_src[inst, 3 * nq + q]
+            o0 = alpha_src[inst, 4 * q]
+            o1 = alpha_src[inst, 4 * q + 1]
+            o2 = alpha_src[inst, 4 * q + 2]
+            o3 = alpha_src[inst, 4 * q + 3]
+            b0 = hmm["output_prob"][o, 4 * q]
+            b1 = hmm["output_prob"][o, 4 * q + 1]
+            b2 = hmm["output_prob"][o, 4 * q + 2]
+            b3 = hmm["output_prob"][o, 4 * q + 3]
+            # reference point of the group: the largest predecessor score, kept finite so that a group
+            # whose predecessors are all unreachable (-inf) gives exp(-inf) = 0 and not exp(nan)
+            m = max(max(max(a1, a2), max(a3, a4)), float32(-3.0e38))
+            e1 = exp(a1 - m)
+            e2 = exp(a2 - m)
+            e3 = exp(a3 - m)
+            e4 = exp(a4 - m)
+            if max(max(o0, o1), max(o2, o3)) - m <= float32(80.0):
+                alpha_dst[inst, 4 * q] = syn4_state(
+                    e1, e2, e3, e4, hmm["ptrans1"][q, 0], hmm["ptrans1"][nq + q, 0],
+                    hmm["ptrans1"][2 * nq + q, 0], hmm["ptrans1"][3 * nq + q, 0], hmm["pstay"][4 * q], o0, m, b0)
+                alpha_dst[inst, 4 * q + 1] = syn4_state(
+                    e1, e2, e3, e4, hmm["ptrans1"][q, 1], hmm["ptrans1"][nq + q, 1],
+                    hmm["ptrans1"][2 * nq + q, 1], hmm["ptrans1"][3 * nq + q, 1], hmm["pstay"][4 * q + 1], o1, m, b1)
+                alpha_dst[inst, 4 * q + 2] = syn4_state(
+                    e1, e2, e3, e4, hmm["ptrans1"][q, 2], hmm["ptrans1"][nq + q, 2],
+                    hmm["ptrans1"][2 * nq + q, 2], hmm["ptrans1"][3 * nq + q, 2], hmm["pstay"][4 * q + 2], o2, m, b2)
+                alpha_dst[inst, 4 * q + 3] = syn4_state(
+                    e1, e2, e3, e4, hmm["ptrans1"][q, 3], hmm["ptrans1"][nq + q, 3],
+                    hmm["ptrans1"][2 * nq + q, 3], hmm["ptrans1"][3 * nq + q, 3], hmm["pstay"][4 * q + 3], o3, m, b3)
+            else:
+                alpha_dst[inst, 4 * q] = syn4_state_wide(
+                    e1, e2, e3, e4, hmm["ptrans1"][q, 0], hmm["ptrans1"][nq + q, 0],
+                    hmm["ptrans1"][2 * nq + q, 0], hmm["ptrans1"][3 * nq + q, 0], hmm["pstay"][4 * q], o0, m, b0)
+                alpha_dst[inst, 4 * q + 1] = syn4_state_wide(
+                    e1, e2, e3, e4, hmm["ptrans1"][q, 1], hmm["ptrans1"][nq + q, 1],
+                    hmm["ptrans1"][2 * nq + q, 1], hmm["ptrans1"][3 * nq + q, 1], hmm["pstay"][4 * q + 1], o1, m, b1)
+                alpha_dst[inst, 4 * q + 2] = syn4_state_wide(
+                    e1, e2, e3, e4, hmm["ptrans1"][q, 2], hmm["ptrans1"][nq + q, 2],
+                    hmm["ptrans1"][2 * nq + q, 2], hmm["ptrans1"][3 * nq + q, 2], hmm["pstay"][4 * q + 2], o2, m, b2)
+                alpha_dst[inst, 4 * q + 3] = syn4_state_wide(
+                    e1, e2, e3, e4, hmm["ptrans1"][q, 3], hmm["ptrans1"][nq + q, 3],
+                    hmm["ptrans1"][2 * nq + q, 3], hmm["ptrans1"][3 * nq + q, 3], hmm["pstay"][4 * q + 3], o3, m, b3)
+
+
+@parpy.jit
+def forward_syn4(hmm, seqs, result, alpha1, alpha2):
+    """The synthetic forward pass with the step written over groups of four states.
+
+    States 4q .. 4q+3 have the same four shift predecessors q, S/4+q, S/2+q, 3S/4+q.  Their scores are
+    referred to the largest of the four once per group, `exp(a_j - m)` is taken once per group, and the
+    transition and stay probabilities enter in linear space (`ptrans1 = exp(trans1)`, `pstay = exp(stay)`):
+    alpha'[4q+u] = m + log(sum_j ptrans1[pred_j, u] * e_j + pstay[4q+u] * exp(alpha[4q+u] - m)) + emission.
+    A group in which some state scores more than e^80 above every predecessor takes a second branch that
+    refers each state to the larger of m and its own score, so no exponential can overflow; unreachable
+    states (-inf) stay -inf.  Same recurrence as `forward_syn` in real arithmetic: 3 exponentials and
+    logarithms per state instead of 6."""
+    parpy.label('inst')
+    for inst in range(seqs["num_instances"]):
+        forward_syn_init(hmm, seqs, alpha1, inst)
+        for t in range(1, seqs["maxlen"]):
+            forward_syn4_step(hmm, seqs, alpha1, alpha2, inst, t)
+        forward_syn_lse(hmm, seqs, result, alpha1, alpha2, inst)
+
+
 # ---------------------------------------------------------------- seeded inputs
 SEED = 1234
 
@@ -347,6 +447,14 @@ def load_reference_model(model_npz, signals_npz):
         data[i, :n] = s["samples"][e - n:e]
     seqs = {"data": data, "lens": lens, "maxlen": int(lens.max()), "num_instances": len(lens)}
     return hmm, seqs
+
+
+def with_linear_tables(hmm):
+    """The model with its transition tables also in linear space (`ptrans1`, `pstay`), as `forward_syn4` reads them."""
+    out = dict(hmm)
+    out["ptrans1"] = np.exp(hmm["trans1"].astype(np.float64)).astype(np.float32)
+    out["pstay"] = np.exp(hmm["stay"].astype(np.float64)).astype(np.float32)
+    return out
 
 
 def to_device(d, device="cuda"):
