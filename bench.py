@@ -1,13 +1,22 @@
 """Benchmark of the compiled hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload hmm7|hmm5|hmm5ref|rowsum|softmax|sddmm|copy]
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+                    [--workload all|hmm7|hmm5|hmm5ref|rowsum|softmax|sddmm|copy] [--form grouped|reference]
 
 A step is one pass of the compiled function over one batch of seeded synthetic
-input that is already resident in HBM.  The default workload is the headline
-one: the 7-mer HMM forward batch (4^7 = 16384 states, 100 reads of 5000..15000
-samples).  One JSON line is printed; it carries the roofline of the dominant
-kernel (algorithmic bytes / measured kernel time against the 8 TB/s HBM peak)
-and a CPU baseline (the C oracle on the host cores, bounded sample).
+input that is already resident in HBM.  The default run (`all`) times the
+headline workload -- the 7-mer HMM forward batch (4^7 = 16384 states, 100 reads
+of 5000..15000 samples) -- and then the other configurations, whose records go
+under `secondary` of the same JSON line.  Every record carries the roofline of
+its dominant kernel (algorithmic bytes or flops / measured kernel time against
+the published peak) and a CPU baseline timed on the host cores (bounded sample).
+
+The HMM forward pass is timed in two forms of the same recurrence, both written
+as ParPy user code in parpy_amd/workloads.py: `grouped` (forward_syn4: the four
+states that share their predecessors are updated together, `value` of the
+headline) and `reference` (forward_syn: one state at a time, the structure of
+the reference's kernel); the figure of the other form is in the record too.
+Results are checked against the oracle outside the timed region.
 """
 import argparse
 import json
@@ -19,6 +28,22 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+FP32_MATRIX_PEAK_TFLOPS = 157.3
+
+OPT_FLAGS = ("opt_vectorize", "opt_lds_rows", "opt_reg_cache", "opt_hoist_invariant", "opt_narrow_index", "opt_unswitch",
+             "opt_gather_transpose", "opt_nontemporal", "opt_lane_split", "opt_drop_barriers", "opt_unswitch_uniform",
+             "opt_offset32", "opt_if_convert", "opt_noalias_scopes", "opt_mfma_sddmm", "opt_expand_short_loops",
+             "opt_guard_bounds")
+
+# Vector-ALU instructions per state and step in the time loop of the generated HMM kernels (counted in the ISA of
+# the kernels as compiled for these shapes: full-rate instructions, and v_exp_f32 / v_log_f32), and the issue times
+# of the two classes measured with register-only microkernels on this part (4 waves per SIMD).  One workgroup of 16
+# waves per read puts S / 256 rows of 64 states on each SIMD.
+VALU_NS = {"full": 1.17, "trans": 3.76}
+HMM_VALU_MIX = {
+    "reference": {"full": 24.0, "trans": 6.0},
+    "grouped": {"full": 16.75, "trans": 3.0},
+}
 
 
 def _events_ms(fn, timed, steps, warmup, torch):
@@ -35,28 +60,60 @@ def _events_ms(fn, timed, steps, warmup, torch):
     return wall, [timed() for _ in range(steps)]
 
 
-def bench_hmm(k, args, torch, parpy, W):
-    import numpy as np
-    hmm, seqs = W.synthetic_hmm(k)
-    S, n = hmm["num_states"], seqs["num_instances"]
-    hd, sd = W.to_device(hmm), W.to_device(seqs)
+def _hbm_roofline(alg_bytes, kernel_ms, workload, default_cfg):
+    gbs = alg_bytes / (kernel_ms * 1e-3) / 1e9
+    traffic, source = _profiled_traffic(workload) if default_cfg else (None, None)
+    return {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
+            "traffic": traffic, "traffic_source": source, "kernel_ms": kernel_ms, "algorithmic_bytes": alg_bytes}
+
+
+def _time_hmm_form(form, hd, sd, n, S, nthreads, args, torch, parpy, W):
     a1 = torch.zeros((n, S), dtype=torch.float32, device="cuda")
     a2 = torch.zeros_like(a1)
     res = torch.zeros(n, dtype=torch.float32, device="cuda")
-    nthreads = min(S, args.state_threads)
-    opts = parpy.par({"inst": parpy.threads(n), "state": parpy.threads(nthreads)})
+    f = W.forward_syn4 if form == "grouped" else W.forward_syn
+    threads = min(nthreads, S // 4) if form == "grouped" else min(nthreads, S)
+    opts = parpy.par({"inst": parpy.threads(n), "state": parpy.threads(threads)})
     _apply_opt_flags(opts, args)
     opts.use_cuda_graphs = bool(args.use_graphs)
-    fn = lambda: W.forward_syn(hd, sd, res, a1, a2, opts=opts)
-    timed = lambda: parpy.time_call(W.forward_syn, hd, sd, res, a1, a2, opts=opts)
+    fn = lambda: f(hd, sd, res, a1, a2, opts=opts)
+    timed = lambda: parpy.time_call(f, hd, sd, res, a1, a2, opts=opts)
     wall, dev = _events_ms(fn, timed, args.steps, args.warmup, torch)
+    dev.sort()
+    return wall, dev[len(dev) // 2], res.cpu().numpy(), threads
+
+
+def bench_hmm(k, args, torch, parpy, W, default_cfg=True):
+    import numpy as np
+    import oracle
+    hmm, seqs = W.synthetic_hmm(k)
+    S, n = hmm["num_states"], seqs["num_instances"]
+    hd, sd = W.to_device(W.with_linear_tables(hmm)), W.to_device(seqs)
     steps_total = int((seqs["lens"] - 1).sum())
+    longest = int(seqs["lens"].max()) - 1
     # per (sequence, step): read alpha (4S) + write alpha (4S) + emission row (4S) + the observation byte
     alg_bytes = (12 * S + 1) * steps_total
-    kernel_ms = float(np.median(dev))
+    other = "reference" if args.form == "grouped" else "grouped"
+    forms = {}
+    for form in (args.form, other):
+        wall, kernel_ms, ll, threads = _time_hmm_form(form, hd, sd, n, S, args.state_threads, args, torch, parpy, W)
+        mix = HMM_VALU_MIX[form]
+        rows_per_simd = S / 256.0
+        bound_ms = longest * rows_per_simd * (mix["full"] * VALU_NS["full"] + mix["trans"] * VALU_NS["trans"]) * 1e-6
+        forms[form] = {"wall": wall, "kernel_ms": kernel_ms, "ll": ll, "threads": threads,
+                       "valu_bound": {"ms": bound_ms, "frac": bound_ms / kernel_ms,
+                                      "model": f"{longest} steps of the longest read x {rows_per_simd:g} rows of 64 states per SIMD x "
+                                               f"({mix['full']} full-rate x {VALU_NS['full']} ns + {mix['trans']} exp/log x {VALU_NS['trans']} ns)"}}
+    # outside the timed region: the shortest reads at full length against the fp64 oracle (what the GPU tests do for all)
+    sub = np.argsort(seqs["lens"])[:6]
+    want = oracle.hmm_syn_forward(hmm, seqs, np.float64, subset=sub)
+    checked = {}
+    for form, r in forms.items():
+        err = float(np.abs(r["ll"][sub].astype(np.float64) - want).max())
+        assert np.all(np.isfinite(r["ll"])) and err < 0.2, f"{form} form of the {k}-mer forward pass is off by {err}"
+        checked[form] = err
     cpu = None
     if not args.no_cpu:
-        import oracle
         sample_steps = args.cpu_steps or (15000 if k <= 5 else 5000)   # about 2 s (5-mer) and 10 s (7-mer) on 16 cores
         t0 = time.perf_counter()
         oracle.hmm_syn_forward(hmm, seqs, np.float32, max_steps=sample_steps)
@@ -65,22 +122,28 @@ def bench_hmm(k, args, torch, parpy, W):
         cpu = {"value": dt * 1e3 * steps_total / done, "unit": "ms/batch", "cores": os.cpu_count(), "kind": "port",
                "sample": f"first {sample_steps} samples of each of the {n} reads with the C oracle "
                          f"(OpenMP over reads), {dt:.1f} s measured, scaled by total steps {steps_total}/{done}"}
-    ll = res.cpu().numpy()
+    main, alt = forms[args.form], forms[other]
+    name = {"grouped": "forward_syn4", "reference": "forward_syn"}
+    roof = _hbm_roofline(alg_bytes, main["kernel_ms"], f"hmm{k}" + ("_grouped" if args.form == "grouped" else ""), default_cfg)
+    roof["valu_bound"] = main["valu_bound"]
+    alt_roof = _hbm_roofline(alg_bytes, alt["kernel_ms"], f"hmm{k}" + ("_grouped" if other == "grouped" else ""), default_cfg)
+    alt_roof["valu_bound"] = alt["valu_bound"]
     return {
         "metric": f"HMM-forward {k}-mer ms/batch + achieved HBM GB/s (% of peak), 1xMI355X",
-        "value": wall, "unit": "ms/batch", "ms_per_step": wall, "higher_is_better": False,
+        "value": main["wall"], "unit": "ms/batch", "ms_per_step": main["wall"], "higher_is_better": False,
         "dtype": "f32",
-        "config": {"workload": f"hmm_forward_{k}mer_synthetic", "states": S, "reads": n, "min_len": 5000,
-                   "max_len": 15000, "total_steps": steps_total, "state_threads": nthreads, "graph_replay": bool(args.use_graphs),
-                   "mean_loglik": float(ll.mean())},
-        "roofline": {"bound": "hbm", "achieved": alg_bytes / (kernel_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": alg_bytes / (kernel_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None,
-                     "kernel_ms": kernel_ms, "algorithmic_bytes": alg_bytes},
+        "config": {"workload": f"hmm_forward_{k}mer_synthetic", "form": f"{args.form} ({name[args.form]})", "states": S, "reads": n,
+                   "min_len": 5000, "max_len": 15000, "total_steps": steps_total, "state_threads": main["threads"],
+                   "graph_replay": bool(args.use_graphs), "mean_loglik": float(main["ll"].mean()),
+                   "checked": f"6 shortest reads at full length against the fp64 oracle, max abs error {checked[args.form]:.3g}"},
+        "roofline": roof,
+        "other_form": {"form": f"{other} ({name[other]})", "ms_per_step": alt["wall"], "state_threads": alt["threads"],
+                       "roofline": alt_roof, "checked_max_abs_error": checked[other]},
         "cpu_baseline": cpu,
     }
 
 
-def bench_hmm_ref(args, torch, parpy, W):
+def bench_hmm_ref(args, torch, parpy, W, default_cfg=True):
     """The reference's own 5-mer model (16 duration layers x 1024 k-mers = 16384 states) on its 100
     recorded reads, tables from tests/golden: the configuration its benchmark validates
     (benchmarks/forward.py:481-518).  Results are checked against the expected log-likelihoods."""
@@ -110,26 +173,30 @@ def bench_hmm_ref(args, torch, parpy, W):
         "value": wall, "unit": "ms/batch", "ms_per_step": wall, "higher_is_better": False, "dtype": "f32",
         "config": {"workload": "hmm_forward_reference_5mer_model", "states": S, "reads": n, "min_len": int(seqs["lens"].min()),
                    "max_len": int(seqs["lens"].max()), "total_steps": steps_total, "state_threads": nthreads,
-                   "mean_loglik": float(got.mean())},
-        "roofline": {"bound": "hbm", "achieved": alg_bytes / (kernel_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": alg_bytes / (kernel_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None,
-                     "kernel_ms": kernel_ms, "algorithmic_bytes": alg_bytes},
+                   "mean_loglik": float(got.mean()),
+                   "checked": f"all {n} reads against the reference's recorded log-likelihoods (atol = rtol = 1e-5), "
+                              f"max abs error {float(np.abs(got - want).max()):.3g}"},
+        "roofline": _hbm_roofline(alg_bytes, kernel_ms, "hmm5ref", default_cfg),
         "cpu_baseline": None,
+        "data": "reference fixtures (tests/golden)",
     }
 
 
-def bench_rowsum(args, torch, parpy, W):
+def bench_rowsum(args, torch, parpy, W, default_cfg=True):
     import numpy as np
     N, M = 1024, 65536
-    args.inner_threads = args.inner_threads or 1024  # one full workgroup per row (any choice from 64 up measures within 5 %)
+    inner = args.inner_threads or 1024  # one full workgroup per row (any choice from 64 up measures within 5 %)
     x = W.make_rowsum(N, M)
     xd = torch.from_numpy(x).cuda()
     out = torch.zeros(N, dtype=torch.float32, device="cuda")
-    opts = parpy.par({"outer": parpy.threads(N), "inner": parpy.threads(args.inner_threads)})
+    opts = parpy.par({"outer": parpy.threads(N), "inner": parpy.threads(inner)})
     _apply_opt_flags(opts, args)
     fn = lambda: W.sum_rows(xd, out, N, opts=opts)
     timed = lambda: parpy.time_call(W.sum_rows, xd, out, N, opts=opts)
     wall, dev = _events_ms(fn, timed, args.steps, args.warmup, torch)
+    want = x.sum(axis=1, dtype=np.float64)
+    err = float(np.abs(out.cpu().numpy() - want).max())
+    assert err < 1e-2, err
     alg = N * M * 4 + N * 4
     kernel_ms = float(np.median(dev))
     cpu = None
@@ -141,45 +208,47 @@ def bench_rowsum(args, torch, parpy, W):
                "sample": "np.sum(x, axis=1) on the full 1024x65536 matrix, mean of 3"}
     return {"metric": "row-sum 1024x65536 f32 ms + achieved HBM GB/s", "value": wall, "unit": "ms/batch", "ms_per_step": wall,
             "higher_is_better": False, "dtype": "f32",
-            "config": {"workload": "rowsum_1024x65536", "inner_threads": args.inner_threads},
-            "roofline": {"bound": "hbm", "achieved": alg / (kernel_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                         "frac": alg / (kernel_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None, "kernel_ms": kernel_ms,
-                         "algorithmic_bytes": alg},
+            "config": {"workload": "rowsum_1024x65536", "inner_threads": inner,
+                       "checked": f"all rows against the fp64 sum, max abs error {err:.3g}"},
+            "roofline": _hbm_roofline(alg, kernel_ms, "rowsum", default_cfg),
             "cpu_baseline": cpu}
 
 
-def bench_softmax(args, torch, parpy, W):
+def bench_softmax(args, torch, parpy, W, default_cfg=True):
     import numpy as np
     N, M = 16384, 4096
-    args.inner_threads = args.inner_threads or 512   # 8 elements (two dwordx4) per thread, 4 workgroups per CU
+    inner = args.inner_threads or 512   # 8 elements (two dwordx4) per thread, 4 workgroups per CU
     x = W.make_softmax(N, M)
     xd = x.cuda()
     out = torch.zeros_like(xd)
-    opts = parpy.par({"N": parpy.threads(N), "M": parpy.threads(args.inner_threads)})
+    opts = parpy.par({"N": parpy.threads(N), "M": parpy.threads(inner)})
     _apply_opt_flags(opts, args)
     fn = lambda: W.softmax(xd, N, M, out, opts=opts)
     timed = lambda: parpy.time_call(W.softmax, xd, N, M, out, opts=opts)
     wall, dev = _events_ms(fn, timed, args.steps, args.warmup, torch)
     alg = 2 * N * M * 4
     kernel_ms = float(np.median(dev))
+    t0 = time.perf_counter()
+    want = torch.softmax(x, 1)
+    cpu_ms = (time.perf_counter() - t0) * 1e3
+    got = out.cpu()
+    rel = float(((got - want).abs() / want).max())
+    assert torch.allclose(got, want, atol=1e-5, rtol=1e-5), rel
     cpu = None
     if not args.no_cpu:
-        t0 = time.perf_counter()
-        for _ in range(3):
-            torch.softmax(x, 1)
-        cpu = {"value": (time.perf_counter() - t0) / 3 * 1e3, "unit": "ms/batch", "cores": torch.get_num_threads(),
-               "kind": "port", "sample": "torch.softmax(x, 1) on the full 16384x4096 matrix, mean of 3"}
+        cpu = {"value": cpu_ms, "unit": "ms/batch", "cores": torch.get_num_threads(),
+               "kind": "port", "sample": "torch.softmax(x, 1) on the full 16384x4096 matrix, one run"}
     return {"metric": "softmax 16384x4096 f32 ms + achieved HBM GB/s", "value": wall, "unit": "ms/batch", "ms_per_step": wall,
             "higher_is_better": False, "dtype": "f32",
-            "config": {"workload": "softmax_16384x4096", "inner_threads": args.inner_threads},
-            "roofline": {"bound": "hbm", "achieved": alg / (kernel_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                         "frac": alg / (kernel_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None, "kernel_ms": kernel_ms,
-                         "algorithmic_bytes": alg},
+            "config": {"workload": "softmax_16384x4096", "inner_threads": inner,
+                       "checked": f"every element against torch.softmax on the CPU, max relative error {rel:.3g}"},
+            "roofline": _hbm_roofline(alg, kernel_ms, "softmax", default_cfg),
             "cpu_baseline": cpu}
 
 
-def bench_sddmm(args, torch, parpy, W):
+def bench_sddmm(args, torch, parpy, W, default_cfg=True):
     import numpy as np
+    import oracle
     A, B, crows, cols, vals = W.make_sddmm()
     nnz = len(cols)
     Ad, Bd = torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda()
@@ -199,24 +268,41 @@ def bench_sddmm(args, torch, parpy, W):
     wall, dev = _events_ms(fn, timed, args.steps, args.warmup, torch)
     kernel_ms = float(np.median(dev))
     flops = 2 * A.shape[1] * nnz
-    alg = A.nbytes + B.nbytes + cols.nbytes + nnz * 8 + vals.nbytes + nnz * 4
+    # what any SDDMM on this mask must move once: A, B, the CSR mask (column indices + row pointers), the result
+    compulsory = A.nbytes + B.nbytes + cols.nbytes + crows.nbytes + nnz * 4
+    # what the COO kernel of the reference's benchmark is handed on top of that: a row index and a value per non-zero
+    coo_bytes = A.nbytes + B.nbytes + cols.nbytes + nnz * 8 + vals.nbytes + nnz * 4
+    rows = rows_d.cpu().numpy()
+    t0 = time.perf_counter()
+    want = oracle.sddmm(A, B, rows, cols)
+    cpu_ms = (time.perf_counter() - t0) * 1e3
+    got = D.cpu().numpy()
+    bad = np.abs(got - want) > 1e-5 + 1e-5 * np.abs(want)
+    assert bad.mean() < 1e-3 and np.abs(got - want).max() < 5e-4, (float(bad.mean()), float(np.abs(got - want).max()))
     cpu = None
     if not args.no_cpu:
-        import oracle
-        rows = rows_d.cpu().numpy()
-        t0 = time.perf_counter()
-        oracle.sddmm(A.astype(np.float32), B.astype(np.float32), rows, cols)
-        cpu = {"value": (time.perf_counter() - t0) * 1e3, "unit": "ms/batch", "cores": 1, "kind": "port",
-               "sample": "chunked NumPy einsum over all non-zeros"}
-    return {"metric": "SDDMM 8192x128x8192 1% ms + GFLOP/s", "value": wall, "unit": "ms/batch", "ms_per_step": wall,
-            "higher_is_better": False, "dtype": "f32", "config": {"workload": "sddmm_8192_k128_1pct", "nnz": nnz, "tpb": args.tpb},
-            "roofline": {"bound": "hbm", "achieved": alg / (kernel_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                         "frac": alg / (kernel_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None, "kernel_ms": kernel_ms,
-                         "algorithmic_bytes": alg, "gflops": flops / (kernel_ms * 1e-3) / 1e9},
+        cpu = {"value": cpu_ms, "unit": "ms/batch", "cores": 1, "kind": "port", "sample": "chunked NumPy einsum over all non-zeros, one run"}
+    tflops = flops / (kernel_ms * 1e-3) / 1e12
+    l2 = _profiled_field("sddmm", "l2_bytes_per_call") if default_cfg else None
+    traffic, source = _profiled_traffic("sddmm") if default_cfg else (None, None)
+    return {"metric": "SDDMM 8192x128x8192 1% ms + TFLOP/s", "value": wall, "unit": "ms/batch", "ms_per_step": wall,
+            "higher_is_better": False, "dtype": "f32",
+            "config": {"workload": "sddmm_8192_k128_1pct", "nnz": nnz, "tpb": args.tpb,
+                       "checked": f"every non-zero against the fp64 oracle: {float(bad.mean()) * 100:.4f} % outside atol = rtol = 1e-5, "
+                                  f"max abs error {float(np.abs(got - want).max()):.3g}"},
+            # the contraction is 0.17 GFLOP of gathered dot products: priced against the fp32 matrix peak as the
+            # workload's definition asks, although the time goes to L2 requests of the row gathers
+            "roofline": {"bound": "mfma", "achieved": tflops, "peak": FP32_MATRIX_PEAK_TFLOPS, "unit": "TFLOP/s",
+                         "frac": tflops / FP32_MATRIX_PEAK_TFLOPS, "traffic": traffic, "traffic_source": source,
+                         "kernel_ms": kernel_ms, "flops": flops,
+                         "hbm_compulsory_bytes": compulsory, "hbm_compulsory_gbs": compulsory / (kernel_ms * 1e-3) / 1e9,
+                         "coo_argument_bytes": coo_bytes,
+                         "l2_bytes_per_call": l2, "l2_gbs": (l2 / (kernel_ms * 1e-3) / 1e9) if l2 else None,
+                         "l2_source": "profiles/sddmm_kernel.md (TCC_REQ_sum x 128 B)" if l2 else None},
             "cpu_baseline": cpu}
 
 
-def bench_copy(args, torch, parpy, W):
+def bench_copy(args, torch, parpy, W, default_cfg=True):
     """Plain device copy of 256 MiB compiled from `out[:] = x[:]`: the calibration kernel for the HBM counters."""
     import numpy as np
     n = 64 * 1024 * 1024
@@ -231,25 +317,30 @@ def bench_copy(args, torch, parpy, W):
     kernel_ms = float(np.median(dev))
     return {"metric": "device copy 256 MiB ms + achieved HBM GB/s", "value": wall, "unit": "ms/batch", "ms_per_step": wall,
             "higher_is_better": False, "dtype": "f32", "config": {"workload": "copy_256MiB"},
-            "roofline": {"bound": "hbm", "achieved": alg / (kernel_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                         "frac": alg / (kernel_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None, "kernel_ms": kernel_ms,
-                         "algorithmic_bytes": alg},
+            "roofline": _hbm_roofline(alg, kernel_ms, "copy", default_cfg),
             "cpu_baseline": None}
 
 
-def _profiled_traffic(name):
-    """HBM bytes per launch from the committed rocprofv3 counter summary of this kernel, or None."""
+def _profiled_field(name, field):
+    """A figure from the committed rocprofv3 counter summary of this kernel (profiles/<name>_kernel.md), or None."""
     import re
     path = os.path.join(ROOT, "profiles", f"{name}_kernel.md")
     try:
-        m = re.search(r"^traffic_bytes_per_launch:\s*(\d+)", open(path).read(), re.M)
+        m = re.search(r"^%s:\s*(\d+)" % re.escape(field), open(path).read(), re.M)
         return int(m.group(1)) if m else None
     except OSError:
         return None
 
 
+def _profiled_traffic(name):
+    """(HBM bytes per launch, where the figure comes from): FETCH_SIZE + WRITE_SIZE of the committed counter run of
+    the same command, not measured in this run."""
+    v = _profiled_field(name, "traffic_bytes_per_launch")
+    return (v, f"profiles/{name}_kernel.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of an earlier run of this command)") if v else (None, None)
+
+
 def _apply_opt_flags(opts, args):
-    for name in ("opt_vectorize", "opt_lds_rows", "opt_reg_cache", "opt_hoist_invariant", "opt_narrow_index", "opt_unswitch", "opt_gather_transpose", "opt_nontemporal", "opt_lane_split", "opt_drop_barriers", "opt_unswitch_uniform", "opt_offset32", "opt_if_convert", "opt_noalias_scopes", "opt_mfma_sddmm"):
+    for name in OPT_FLAGS:
         v = getattr(args, name)
         if v is not None:
             setattr(opts, name, bool(v))
@@ -262,14 +353,16 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="hmm7", choices=["hmm7", "hmm5", "hmm5ref", "rowsum", "softmax", "sddmm", "copy"])
+    ap.add_argument("--workload", default="all", choices=["all", "hmm7", "hmm5", "hmm5ref", "rowsum", "softmax", "sddmm", "copy"])
+    ap.add_argument("--form", default="grouped", choices=["grouped", "reference"],
+                    help="which statement of the HMM step is the record's value (the other is timed beside it)")
     ap.add_argument("--state-threads", type=int, default=1024)
     ap.add_argument("--use-graphs", type=int, default=0, help="replay the launches of a run from a HIP graph (host-hoisted time loops)")
     ap.add_argument("--inner-threads", type=int, default=None)
     ap.add_argument("--tpb", type=int, default=256)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-steps", type=int, default=0, help="samples per read for the HMM CPU baseline")
-    for name in ("opt_vectorize", "opt_lds_rows", "opt_reg_cache", "opt_hoist_invariant", "opt_narrow_index", "opt_unswitch", "opt_gather_transpose", "opt_nontemporal", "opt_lane_split", "opt_drop_barriers", "opt_unswitch_uniform", "opt_offset32", "opt_if_convert", "opt_noalias_scopes", "opt_mfma_sddmm"):
+    for name in OPT_FLAGS:
         ap.add_argument("--" + name.replace("_", "-"), dest=name, type=int, default=None)
     ap.add_argument("--reg-budget", type=int, default=0)
     args = ap.parse_args()
@@ -285,26 +378,30 @@ def main():
     import parpy_amd as parpy
     from parpy_amd import workloads as W
 
-    if args.workload == "hmm7":
-        r = bench_hmm(7, args, torch, parpy, W)
-    elif args.workload == "hmm5":
-        r = bench_hmm(5, args, torch, parpy, W)
-    elif args.workload == "hmm5ref":
-        r = bench_hmm_ref(args, torch, parpy, W)
-    elif args.workload == "rowsum":
-        r = bench_rowsum(args, torch, parpy, W)
-    elif args.workload == "softmax":
-        r = bench_softmax(args, torch, parpy, W)
-    elif args.workload == "copy":
-        r = bench_copy(args, torch, parpy, W)
+    default_cfg = not any(getattr(args, n) is not None for n in OPT_FLAGS) and not args.reg_budget
+    runners = {
+        "hmm7": lambda: bench_hmm(7, args, torch, parpy, W, default_cfg),
+        "hmm5": lambda: bench_hmm(5, args, torch, parpy, W, default_cfg),
+        "hmm5ref": lambda: bench_hmm_ref(args, torch, parpy, W, default_cfg),
+        "rowsum": lambda: bench_rowsum(args, torch, parpy, W, default_cfg),
+        "softmax": lambda: bench_softmax(args, torch, parpy, W, default_cfg),
+        "sddmm": lambda: bench_sddmm(args, torch, parpy, W, default_cfg),
+        "copy": lambda: bench_copy(args, torch, parpy, W, default_cfg),
+    }
+    common = {"n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "scaling": "weak", "vs_baseline": None}
+    if args.workload == "all":
+        r = runners["hmm7"]()
+        r.update(common)
+        r.setdefault("data", "synthetic")
+        r["secondary"] = []
+        for w in ("hmm5", "hmm5ref", "rowsum", "softmax", "sddmm"):
+            s = runners[w]()
+            s.setdefault("data", "synthetic")
+            r["secondary"].append(s)
     else:
-        r = bench_sddmm(args, torch, parpy, W)
-    default_cfg = not any(getattr(args, n) is not None for n in ("opt_vectorize", "opt_lds_rows", "opt_reg_cache",
-                                                                 "opt_hoist_invariant", "opt_narrow_index", "opt_unswitch", "opt_gather_transpose", "opt_nontemporal", "opt_lane_split", "opt_drop_barriers", "opt_unswitch_uniform", "opt_offset32", "opt_if_convert", "opt_noalias_scopes", "opt_mfma_sddmm"))
-    if default_cfg and not args.reg_budget:
-        r["roofline"]["traffic"] = _profiled_traffic(args.workload)
-    r.update({"n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "scaling": "weak", "vs_baseline": None,
-              "data": "reference fixtures (tests/golden)" if args.workload == "hmm5ref" else "synthetic"})
+        r = runners[args.workload]()
+        r.update(common)
+        r.setdefault("data", "synthetic")
     print(json.dumps(r))
 
 

@@ -214,6 +214,74 @@ def test_hmm_single_block_is_one_kernel_with_lds_rows():
     assert "lds_alpha" not in s0 and "inv_hmm" not in s0
 
 
+def test_grouped_hmm_step_expands_its_state_loop_and_runs_to_the_read_length():
+    """`forward_syn4`: the tables of all four states of a group are hoisted (the helper calls are inlined and the
+    indices depend on the group alone), the time loop runs to min(maxlen, len) without the per-group test, the
+    thread keeps the strided group mapping (an iteration already owns 16 bytes), maxima of loaded values are
+    single instructions."""
+    hmm, seqs, args = _hmm_args(5)
+    args = [W.with_linear_tables(args[0])] + args[1:]
+    o = opts_for({'inst': parpy.threads(4), 'state': parpy.threads(64)})
+    s = compiles(parpy.print_compiled(W.forward_syn4, args, o))
+    assert launch(s) == [("1", "4", "1", "64", "1", "1")]
+    assert len(re.findall(r"float inv_hmm_ptrans1_\d+\[4\];", s)) == 16 and len(re.findall(r"float inv_hmm_pstay_\d+\[4\];", s)) == 4
+    assert re.search(r"int64_t t_end_\d+ = parpy_min<int64_t>\(", s) and re.search(r"for \(int t_\d+ = 1; t_\d+ < t_end_\d+;", s)
+    step = s[s.index("for (int t_"):].split("__syncthreads")[0]
+    assert "seqs_lens" not in step                                   # the test on the read length is gone from the step
+    assert not re.search(r"(?<!inv_)hmm_ptrans1_\d+\[", step) and "hmm_pstay_" not in step.replace("inv_hmm_pstay_", "")
+    assert re.search(r"int q_\d+ = \(\(int\)threadIdx.x \+ q_\d+_k \* 64\);", step)   # groups strided over the threads
+    assert "parpy_fmax3c(" in step and "fmaxf(" not in step
+    s0 = compiles(parpy.print_compiled(W.forward_syn4, args, opts_for({'inst': parpy.threads(4), 'state': parpy.threads(64)},
+                                                                       opt_guard_bounds=False)))
+    assert "t_end_" not in s0 and "seqs_lens" in s0[s0.index("for (int t_"):].split("__syncthreads")[0]
+
+
+def test_short_counted_loops_inside_an_iteration_are_expanded():
+    @parpy.jit
+    def taps(x, w, out, N):
+        parpy.label('i')
+        for i in range(N):
+            t = parpy.operators.float32(0.0)
+            for u in range(3):
+                t = t + w[u] * x[i + u]
+            out[i] = t
+    x, w, out = np.zeros(1026, dtype=np.float32), np.zeros(3, dtype=np.float32), np.zeros(1024, dtype=np.float32)
+    s = compiles(parpy.print_compiled(taps, [x, w, out, 1024], opts_for({'i': parpy.threads(1024)})))
+    assert "for (int u_" not in s and "for (int64_t u_" not in s
+    s0 = compiles(parpy.print_compiled(taps, [x, w, out, 1024], opts_for({'i': parpy.threads(1024)}, opt_expand_short_loops=False)))
+    assert re.search(r"for \(int(64_t)? u_\d+ = 0; u_\d+ < 3;", s0)
+
+
+def test_loop_bound_from_guard_needs_every_effect_under_the_guard():
+    """A statement outside the `t < n[i]` test that stores to memory keeps the loop as written."""
+    @parpy.jit
+    def walk(x, n, out, cnt, N, T):
+        parpy.label('i')
+        for i in range(N):
+            for t in range(T):
+                parpy.label('j')
+                for j in range(64):
+                    if t < n[i]:
+                        out[i, j] = out[i, j] + x[i, t]
+    @parpy.jit
+    def walk_and_count(x, n, out, cnt, N, T):
+        parpy.label('i')
+        for i in range(N):
+            for t in range(T):
+                parpy.label('j')
+                for j in range(64):
+                    cnt[i, j] = cnt[i, j] + 1
+                    if t < n[i]:
+                        out[i, j] = out[i, j] + x[i, t]
+    x, n = np.zeros((8, 100), dtype=np.float32), np.zeros(8, dtype=np.int64)
+    out, cnt = np.zeros((8, 64), dtype=np.float32), np.zeros((8, 64), dtype=np.int64)
+    o = opts_for({'i': parpy.threads(8), 'j': parpy.threads(64)})
+    s = compiles(parpy.print_compiled(walk, [x, n, out, cnt, 8, 100], o))
+    assert re.search(r"t_end_\d+ = parpy_min<int64_t>\(\(int64_t\)\(100\), ", s)
+    s = compiles(parpy.print_compiled(walk_and_count, [x, n, out, cnt, 8, 100], o))
+    assert "t_end_" not in s
+
+
 def test_noalias_scope_wraps_the_step_body_when_aliases_never_coincide():
     hmm, seqs, args = _hmm_args(4)
     o = opts_for({'inst': parpy.threads(4), 'state': parpy.threads(256)}, opt_noalias_scopes=True)
