@@ -416,6 +416,98 @@ struct Pass {
     return out;
   }
 
+  // ================================================================ loads that depend on the step counter alone
+  // Inside a sequential loop that a workgroup walks step by step (a barrier per step), `o = data[i, t]`
+  // is needed at the very start of step t and everything else of the step hangs on it (it selects the
+  // emission row).  The array is never written and the address is a function of t and of values that
+  // do not change in the loop, so the load for step t + 1 is issued at the start of step t into a second
+  // variable: its latency passes behind a whole step of work.  The index must be provably in bounds
+  // over the static range of the loop (the last iteration re-reads its own element instead of t + 1).
+  Stmts prefetch_counter_loads(const Stmts& ss, RangeEnv env) {
+    std::set<Name> params = param_names();
+    std::set<Name> written = written_arrays();
+    Stmts out;
+    for (size_t pos = 0; pos < ss.size(); ++pos) {
+      const S& s = ss[pos];
+      bool seq = s->k == Stmt::For && s->map.k == GpuMap::None && !s->unroll && s->step == 1 && s->lo->k == Expr::Int;
+      // static upper bound of the loop: a literal, or a variable defined just before as min(literal, ...)
+      int64_t HI = -1;
+      if (seq) {
+        if (s->hi->k == Expr::Int) HI = s->hi->iv;
+        else if (s->hi->k == Expr::Var)
+          for (size_t b = 0; b < out.size(); ++b)
+            if (out[b]->k == Stmt::Def && out[b]->id == s->hi->name && out[b]->expr->k == Expr::BinOpE && out[b]->expr->bop == BinOp::Min) {
+              for (auto& a : out[b]->expr->args) if (a->k == Expr::Int) HI = a->iv;
+            }
+      }
+      bool barrier_inside = false;
+      if (seq) visit_stmts(s->body, [&](const S& c) { if (c->k == Stmt::Sync || c->k == Stmt::SyncPoint) barrier_inside = true; });
+      if (seq && HI > s->lo->iv && barrier_inside) {
+        std::set<Name> varying{s->id}, reassigned;
+        visit_stmts(s->body, [&](const S& c) {
+          if (c->k == Stmt::Def || c->k == Stmt::For) varying.insert(c->id);
+          if (c->k == Stmt::Assign && c->dst->k == Expr::Var) { varying.insert(c->dst->name); reassigned.insert(c->dst->name); }
+        });
+        varying.erase(s->id);
+        RangeEnv le = env;
+        Interval tr;
+        tr.known = true;
+        tr.lo = s->lo->iv;
+        tr.hi = HI - 1;
+        le[s->id] = tr;
+        Stmts pre, body;
+        for (auto& c : s->body) {
+          E ld = c->k == Stmt::Def && c->expr ? strip_converts(c->expr) : E();
+          bool ok = ld && ld->k == Expr::Index && c->ty.is_scalar() && !reassigned.count(c->id) && ld->args[0]->k == Expr::Var &&
+                    params.count(ld->args[0]->name) && !written.count(ld->args[0]->name) && !ld->dim_shape.empty() && mentions(ld->args[1], s->id);
+          if (ok) {
+            visit_exprs(ld->args[1], [&](const E& x) {
+              if (x->k == Expr::Var && varying.count(x->name)) ok = false;
+              if (x->k == Expr::Index || x->k == Expr::RegElem || x->k == Expr::ThreadIdx || x->k == Expr::Call || x->k == Expr::Raw) ok = false;
+            });
+          }
+          if (ok) {
+            int64_t numel = 1;
+            for (auto d : ld->dim_shape) numel *= d;
+            Interval r = expr_range(ld->args[1], le);
+            ok = r.known && r.lo >= 0 && r.hi < numel;
+          }
+          if (!ok) { body.push_back(c); continue; }
+          Type ity = s->lo->ty;
+          auto at = [&](const E& t) {
+            std::map<Name, E> m{{s->id, t}};
+            return subst_vars(c->expr, m);
+          };
+          Name nxt = gen.fresh(c->id.s + "_next");
+          pre.push_back(mk_def(nxt, c->ty, at(s->lo), c->i));
+          body.push_back(mk_def(c->id, c->ty, mk_var(nxt, c->ty), c->i));
+          E t1 = mk_binop(BinOp::Min, mk_binop(BinOp::Add, mk_var(s->id, ity), mk_int(1, ity.sz), ity), mk_int(HI - 1, ity.sz), ity);
+          body.push_back(mk_assign(mk_var(nxt, c->ty), at(t1), c->i));
+        }
+        if (!pre.empty()) {
+          for (auto& d : pre) out.push_back(d);
+          auto r = clone(s);
+          r->body = body;
+          out.push_back(r);
+          continue;
+        }
+      }
+      auto r = clone(s);
+      RangeEnv ne = env;
+      if (s->k == Stmt::For && s->lo && s->hi && s->lo->k == Expr::Int && s->hi->k == Expr::Int && s->hi->iv > s->lo->iv) {
+        Interval v;
+        v.known = true;
+        v.lo = s->lo->iv;
+        v.hi = s->hi->iv - 1;
+        ne[s->id] = v;
+      }
+      r->body = prefetch_counter_loads(s->body, ne);
+      r->els = prefetch_counter_loads(s->els, ne);
+      out.push_back(r);
+    }
+    return out;
+  }
+
   // ================================================================ conditions no iteration changes
   // A parallel loop whose whole body is `if (c) A else B`, with c the same for every iteration (it
   // mentions neither the loop variable nor anything the body defines or assigns, and loads only from
@@ -981,9 +1073,9 @@ struct Pass {
   int64_t reg_budget() const {
     if (opts.reg_budget > 0) return opts.reg_budget;
     int64_t threads = k.block.x * k.block.y * k.block.z;
-    // a 1024-thread block leaves 128 VGPRs per lane; 96 cached values plus the
-    // working set still fit without spilling (measured on the HMM kernels)
-    return threads <= 256 ? 192 : threads <= 512 ? 128 : 96;
+    // a 1024-thread block leaves 128 VGPRs per lane; 88 cached values plus the
+    // working set fit without spilling (measured on the HMM kernels; 96 spills a few)
+    return threads <= 256 ? 192 : threads <= 512 ? 128 : 88;
   }
 
   // hoist out of the sequential loop `seq` (a statement of `parent`)
@@ -2295,6 +2387,7 @@ void hip_optimize(Program& p, const Options& opts, NameGen& gen) {
     if (opts.opt_mfma_sddmm) k.body = pass.mfma_dot(k.body);
     if (opts.opt_expand_short_loops) k.body = pass.expand_short_loops(k.body, false);
     if (opts.opt_guard_bounds) k.body = pass.guards_to_bounds(k.body);
+    if (opts.opt_prefetch_steps) k.body = pass.prefetch_counter_loads(k.body, RangeEnv());
     if (opts.opt_unswitch_uniform) k.body = pass.hoist_uniform_conditions(k.body);
     if (opts.opt_if_convert) k.body = pass.if_convert(k.body);
     if (opts.opt_lds_rows) pass.lds_rows();
