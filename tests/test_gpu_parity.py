@@ -137,10 +137,14 @@ def test_softmax_full_size_and_without_register_caching():
     x = W.make_softmax(N, M)
     xd = x.cuda()
     want = torch.softmax(x, 1)
-    for kw in ({}, {"opt_reg_cache": False, "opt_vectorize": False}):
+    # 512 threads per row is the specialisation the benchmark times; 1024 and 64 are other shapes of the same kernel
+    for threads, kw in ((512, {}), (1024, {}), (64, {}), (1024, {"opt_reg_cache": False, "opt_vectorize": False})):
         out = torch.zeros_like(xd)
-        W.softmax(xd, N, M, out, opts=opts_for({'N': parpy.threads(N), 'M': parpy.threads(1024)}, **kw))
+        W.softmax(xd, N, M, out, opts=opts_for({'N': parpy.threads(N), 'M': parpy.threads(threads)}, **kw))
         got = out.cpu()
+        rel = float(((got - want).abs() / want).max())
+        print(f"softmax 16384x4096 on {threads} threads per row {kw}: max relative error {rel:.3g}")
+        assert rel < 1e-5                                   # north_star: 1e-5 relative (measured 8e-7)
         assert torch.allclose(got, want, atol=1e-5, rtol=1e-5)
         assert torch.allclose(got.sum(1), torch.ones(N), atol=1e-5)
 
@@ -404,6 +408,18 @@ def test_forward_grouped_wide_score_ranges_take_the_second_branch():
     assert np.abs(got - w64).max() < 1e-3
 
 
+@pytest.mark.parametrize("bounds", [True, False], ids=["loop-bound", "tested-every-step"])
+def test_forward_batch_larger_than_the_chip_with_ragged_lengths(bounds):
+    """1000 reads of 2..400 samples (more workgroups than compute units): a workgroup whose time loop runs to its
+    read's length gives the same results as one that walks to the longest read testing `t < len` at every step."""
+    hmm, seqs = W.synthetic_hmm(5, n_inst=1000, min_len=2, max_len=400, seed=5)
+    want = oracle.hmm_syn_forward(hmm, seqs, np.float32)
+    got, _, _ = _run_synthetic(hmm, seqs, 1024, opt_guard_bounds=bounds)
+    assert np.allclose(got, want, atol=1e-5, rtol=1e-5), np.abs(got - want).max()
+    got, _, _ = _run_grouped(hmm, seqs, 256, opt_guard_bounds=bounds)
+    assert np.allclose(got, want, atol=1e-5, rtol=1e-5), np.abs(got - want).max()
+
+
 def test_forward_all_states_unreachable_gives_neg_inf():
     hmm, seqs = W.synthetic_hmm(4, n_inst=4, min_len=5, max_len=20)
     hmm["initial_prob"][:] = -np.inf
@@ -434,9 +450,13 @@ def test_sddmm(n, k, density, flags):
     want = oracle.sddmm(A, B, rows, cols, vals, alpha=1.5, beta=2.0)
     got = D.cpu().numpy()
     bad = np.abs(got - want) > 1e-5 + 1e-5 * np.abs(want)
-    # the reference's own criterion (benchmarks/sddmm.py:93-103): fatal from 5 elements and 5 %
-    assert bad.sum() < 5 or bad.mean() < 0.05, (bad.sum(), np.abs(got - want).max())
-    assert np.abs(got - want).max() < 5e-4
+    err = float(np.abs(got - want).max())
+    print(f"sddmm n={n} k={k} {flags}: {int(bad.sum())} of {nnz} elements outside atol = rtol = 1e-5 of the fp64 oracle, max abs error {err:.3g}")
+    # Measured: no element outside the tolerance in any configuration, max abs error 8.6e-6 at full size (sums of
+    # 128 products of magnitude ~1).  The reference itself only calls a mismatch fatal from 5 elements and 5 %
+    # (benchmarks/sddmm.py:93-103); the bound here is one element in ten thousand.
+    assert bad.mean() <= 1e-4, (int(bad.sum()), err)
+    assert err < 5e-5
 
 
 @pytest.mark.parametrize("k", [96, 50])
