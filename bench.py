@@ -76,6 +76,7 @@ def _time_hmm_form(form, hd, sd, n, S, nthreads, args, torch, parpy, W):
     opts = parpy.par({"inst": parpy.threads(n), "state": parpy.threads(threads)})
     _apply_opt_flags(opts, args)
     opts.use_cuda_graphs = bool(args.use_graphs)
+    opts.persistent_loops = bool(args.persistent)
     fn = lambda: f(hd, sd, res, a1, a2, opts=opts)
     timed = lambda: parpy.time_call(f, hd, sd, res, a1, a2, opts=opts)
     wall, dev = _events_ms(fn, timed, args.steps, args.warmup, torch)
@@ -358,6 +359,7 @@ def main():
                     help="which statement of the HMM step is the record's value (the other is timed beside it)")
     ap.add_argument("--state-threads", type=int, default=1024)
     ap.add_argument("--use-graphs", type=int, default=0, help="replay the launches of a run from a HIP graph (host-hoisted time loops)")
+    ap.add_argument("--persistent", type=int, default=0, help="run host-hoisted time loops inside one kernel when the grid fits the device")
     ap.add_argument("--inner-threads", type=int, default=None)
     ap.add_argument("--tpb", type=int, default=256)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")

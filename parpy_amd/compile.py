@@ -174,6 +174,7 @@ def get_wrapper(name, key, plan_text, opts):
     wrapper.plan = plan
     wrapper.launch_count = lambda: lib.parpy_hip_plan_launch_count(plan)
     wrapper.graph_replays = lambda: lib.parpy_hip_plan_graph_replays(plan)
+    wrapper.persistent_launches = lambda: lib.parpy_hip_plan_persistent_launches(plan)
     return wrapper
 
 

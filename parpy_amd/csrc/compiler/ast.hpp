@@ -253,6 +253,7 @@ struct Stmt {
     Alloc,      // id = device allocation of iv elements of type ty.sz
     Free,       // free id
     Launch,     // kernel launch: fname, grid/block, args
+    PersistentLaunch,  // one launch of kernel fname that runs a whole host loop of launches (kept in body) with device-wide barriers
     Scope,      // { body }; with args: the pointer variables in args do not alias each other inside
     WaveReduce, // id = wave_reduce<bop>(id)
     LdsDecl,    // __shared__ ty.sz id[iv]
@@ -362,6 +363,7 @@ struct Options {  // src/option.rs:14-108
   bool debug_print = false;
   Backend backend = Backend::Hip;
   bool use_graphs = false;
+  bool persistent_loops = false;  // host loops of launches run inside one kernel, steps separated by a barrier over all workgroups
   bool has_force_int = false, has_force_float = false;
   ElemSize force_int = ElemSize::I64, force_float = ElemSize::F64;
   std::vector<std::string> includes;
@@ -407,6 +409,7 @@ struct Kernel {
   bool aligned_params = false;  // every pointer argument is 16-byte aligned (checked by the caller)
   bool cached_stores = false;   // what this kernel writes is read by the next one: no non-temporal stores
   bool opaque_body = false;     // the body is a call of a device helper: parameters are described by the creator
+  bool no_restrict = false;     // workgroups exchange data through the parameters during the kernel: no no-alias promise
 };
 
 struct Program {

@@ -2374,6 +2374,113 @@ struct Coarsen {
   }
 };
 
+// ================================================================ host loops of launches inside one kernel
+// A sequential loop that had to move to the host because its steps need all workgroups to meet
+// (`for t: launch step(t)`) pays the fixed cost of a dependent launch per step -- several microseconds
+// on the device, more than the step itself when the launch is small.  With `persistent_loops` the loop
+// also exists as one kernel: the bodies of the step kernels in a `for t` loop, each followed by a barrier
+// over all workgroups of the launch (a counter in device memory, release / acquire fences at device
+// scope, a bounded wait).  The runtime uses that kernel only when the whole grid fits on the device at
+// once -- otherwise workgroups would wait for others that cannot start -- and runs the loop of launches
+// as before when it does not.
+struct PersistentLoops {
+  Program& p;
+  const Options& opts;
+  NameGen& gen;
+  ElemSize isz;
+
+  PersistentLoops(Program& prog, const Options& o, NameGen& g) : p(prog), opts(o), gen(g), isz(o.int_size()) {}
+
+  Kernel* find(const std::string& name) {
+    for (auto& k : p.kernels)
+      if (k.name == name) return &k;
+    return nullptr;
+  }
+
+  S fuse(const S& loop) {
+    if (!(loop->k == Stmt::For && loop->map.k == GpuMap::None && loop->step == 1 && !loop->body.empty())) return S();
+    std::vector<Kernel*> ks;
+    for (auto& l : loop->body) {
+      if (l->k != Stmt::Launch) return S();
+      Kernel* k = find(l->fname);
+      if (!k || k->opaque_body) return S();
+      // the argument of every parameter must be the host variable of the same name (how launches are generated)
+      for (size_t i = 0; i < k->params.size(); ++i)
+        if (!(l->args[i]->k == Expr::Var && l->args[i]->name == k->params[i].id)) return S();
+      ks.push_back(k);
+    }
+    const Kernel& k0 = *ks[0];
+    for (auto* k : ks)
+      if (k->grid.x != k0.grid.x || k->grid.y != k0.grid.y || k->grid.z != k0.grid.z || k->block.x != k0.block.x ||
+          k->block.y != k0.block.y || k->block.z != k0.block.z)
+        return S();
+    int64_t nblocks = k0.grid.x * k0.grid.y * k0.grid.z;
+    // the barrier counter runs up to (number of barriers) x (number of workgroups) in 32 bits
+    if (loop->lo->k != Expr::Int || loop->hi->k != Expr::Int) return S();
+    int64_t trips = loop->hi->iv - loop->lo->iv;
+    if (trips < 2 || trips * (int64_t)ks.size() * nblocks >= (int64_t(1) << 32)) return S();
+    Kernel f;
+    f.name = p.name + "_steps_" + std::to_string(gen.next++);
+    f.grid = k0.grid;
+    f.block = k0.block;
+    f.cached_stores = true;
+    f.no_restrict = true;
+    f.aligned_params = k0.aligned_params;
+    std::map<Name, size_t> seen;
+    for (auto* k : ks)
+      for (auto& q : k->params) {
+        if (q.id == loop->id) continue;
+        auto it = seen.find(q.id);
+        if (it == seen.end()) { seen[q.id] = f.params.size(); f.params.push_back(q); }
+        else if (!q.read_only) f.params[it->second].read_only = false;
+      }
+    Type u32 = Type::scalar(ElemSize::U32);
+    KernelParam counter, status, limit;
+    counter.id = gen.fresh("parpy_bar_counter"); counter.ty = Type::pointer(ElemSize::U32);
+    status.id = gen.fresh("parpy_bar_status"); status.ty = Type::pointer(ElemSize::U32);
+    limit.id = gen.fresh("parpy_bar_limit"); limit.ty = u32;
+    std::string bar = "if (!parpy_grid_barrier(" + counter.id.str() + ", " + status.id.str() + ", " + std::to_string(nblocks) +
+                      "u, parpy_bar_epoch, " + limit.id.str() + ")) return;";
+    Stmts step;
+    for (auto* k : ks) {
+      step.push_back(mk_scope(k->body));
+      step.push_back(mk_rawstmt(bar));
+    }
+    auto t = clone(loop);
+    t->body = step;
+    f.body = {mk_rawstmt("unsigned parpy_bar_epoch = 0;"), S(t)};
+    auto l = std::make_shared<Stmt>();
+    l->k = Stmt::PersistentLaunch;
+    l->fname = f.name;
+    l->grid = f.grid;
+    l->block = f.block;
+    l->i = loop->i;
+    for (auto& q : f.params) l->args.push_back(mk_var(q.id, q.ty));
+    l->body = {loop};
+    f.params.push_back(counter);
+    f.params.push_back(status);
+    f.params.push_back(limit);
+    p.kernels.push_back(f);
+    return l;
+  }
+
+  Stmts walk(const Stmts& ss) {
+    Stmts out;
+    for (auto& s : ss) {
+      if (S f = fuse(s)) { out.push_back(f); continue; }
+      auto r = clone(s);
+      if (s->k == Stmt::For || s->k == Stmt::While || s->k == Stmt::If) {
+        r->body = walk(s->body);
+        r->els = walk(s->els);
+      }
+      out.push_back(r);
+    }
+    return out;
+  }
+
+  void run() { p.host = walk(p.host); }
+};
+
 }  // namespace
 
 void hip_optimize(Program& p, const Options& opts, NameGen& gen) {
@@ -2400,6 +2507,7 @@ void hip_optimize(Program& p, const Options& opts, NameGen& gen) {
     pass.mark_read_only();
     k.aligned_params = opts.assume_aligned;
   }
+  if (opts.persistent_loops) PersistentLoops(p, opts, gen).run();
 }
 
 }  // namespace parpy

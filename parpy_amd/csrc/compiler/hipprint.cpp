@@ -175,6 +175,31 @@ template <class T> __device__ __forceinline__ T parpy_sum8(T v) {
   v = v + parpy_dpp<0x141>(v);  // the other quad of the 8-lane half row
   return v;
 }
+// Barrier over all workgroups of a launch whose whole grid is resident on the device.  The kernels that use it
+// load and store what they exchange at device scope, so no cache has to be written back or emptied here: every
+// wave waits until its own memory operations have completed, the workgroup's first thread counts the workgroup in
+// and waits until the counter shows that all have arrived (the counter is never reset: call number e waits for
+// e * nblocks).  The wait is bounded: after `limit` polls, or when another workgroup has given up, the status word
+// is set and false is returned to the whole workgroup, which leaves the kernel.
+__device__ __forceinline__ bool parpy_grid_barrier(unsigned* counter, unsigned* status, unsigned nblocks, unsigned& epoch, unsigned limit) {
+  __shared__ unsigned parpy_bar_ok;
+  __builtin_amdgcn_s_waitcnt(0x0070);   // vmcnt(0) lgkmcnt(0): this wave's loads and stores are done
+  __syncthreads();
+  epoch += 1;
+  if (threadIdx.x == 0 && threadIdx.y == 0 && threadIdx.z == 0) {
+    const unsigned target = epoch * nblocks;
+    __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    unsigned ok = 1, polls = 0;
+    while (__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) {
+      if (polls++ >= limit || __hip_atomic_load(status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) { ok = 0; break; }
+      __builtin_amdgcn_s_sleep(1);
+    }
+    if (!ok) __hip_atomic_store(status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    parpy_bar_ok = ok;
+  }
+  __syncthreads();
+  return parpy_bar_ok != 0;
+}
 typedef float parpy_f32x4 __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ int parpy_lane_id() { return (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)); }
 // dst[c][r] = src[r][c] for a ROWS x COLS matrix in 64 x 64 tiles: a 256-thread workgroup reads
@@ -325,6 +350,16 @@ struct DevicePrinter {
     if (sz == ElemSize::F64) return base;
     if (fast) return std::string("__") + base + "f";
     return std::string(base) + "f";
+  }
+
+  // accesses that must be coherent across the device: global elements of arrays that a kernel with
+  // device-wide barriers may write (everything that is not a read-only parameter)
+  bool as_lvalue = false;
+  bool exchanged(const E& e) const {
+    if (!kernel || !kernel->no_restrict || e->k != Expr::Index) return false;
+    const E& base = e->args[0];
+    if (base->ty.mem == Mem::LDS || elem_bytes(e->ty.sz) < 4) return false;
+    return !read_only_param(base);
   }
 
   // fp32 values that come straight from memory (a load, or a variable that only names one): what the compiler
@@ -480,6 +515,11 @@ struct DevicePrinter {
         }
         for (auto& n : assumed) ranges.erase(n);
         for (auto& kv : narrowed) ranges[kv.first] = kv.second;
+        // Workgroups of this kernel exchange data through global memory between device-wide barriers: what is
+        // not read-only is loaded and stored at device scope (past the caches that are private to a compute
+        // unit or a die), so the barrier itself needs no cache write-back or invalidation.
+        if (exchanged(e) && !as_lvalue)
+          return "__hip_atomic_load(&" + out + ", __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)";
         return out;
       }
       case Expr::AddrOf: return "(&" + pexpr(e->args[0]) + "[" + pexpr(e->args[1]) + "])";
@@ -686,6 +726,14 @@ struct DevicePrinter {
           os << ind(n) << "__builtin_nontemporal_store((" << elem_ctype(s->dst->ty.sz) << ")" << paren(rhs) << ", &" << pexpr(s->dst) << ");\n";
           break;
         }
+        if (s->dst->k == Expr::Index && exchanged(s->dst)) {
+          as_lvalue = true;
+          std::string lhs = pexpr(s->dst);
+          as_lvalue = false;
+          os << ind(n) << "__hip_atomic_store(&" << lhs << ", (" << elem_ctype(s->dst->ty.sz) << ")" << paren(rhs)
+             << ", __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);\n";
+          break;
+        }
         os << ind(n) << pexpr(s->dst) << " = " << rhs << ";\n";
         break;
       }
@@ -794,7 +842,8 @@ struct DevicePrinter {
     for (size_t i = 0; i < k.params.size(); ++i) {
       const auto& p = k.params[i];
       out << (i ? ", " : "");
-      if (p.ty.k == Type::Pointer) out << (p.read_only ? "const " : "") << elem_ctype(p.ty.sz) << "* __restrict__ " << p.id.str();
+      if (p.ty.k == Type::Pointer)
+        out << (p.read_only ? "const " : "") << elem_ctype(p.ty.sz) << (k.no_restrict && !p.read_only ? "* " : "* __restrict__ ") << p.id.str();
       else out << elem_ctype(p.ty.sz) << " " << p.id.str();
     }
     out << ") {\n";
@@ -869,6 +918,18 @@ struct PlanPrinter {
           os << "))";
           break;
         }
+        case Stmt::PersistentLaunch: {
+          size_t idx = 0;
+          for (; idx < p.kernels.size(); ++idx)
+            if (p.kernels[idx].name == s->fname) break;
+          os << "(persist " << idx << " " << s->grid.x << " " << s->grid.y << " " << s->grid.z << " " << s->block.x << " "
+             << s->block.y << " " << s->block.z << " (args";
+          for (auto& a : s->args) os << " " << hexpr(a);
+          os << ") (body ";
+          stmts(s->body);
+          os << "))";
+          break;
+        }
         case Stmt::For:
           os << "(for " << sx_quote(s->id.str()) << " " << hexpr(s->lo) << " " << hexpr(s->hi) << " " << s->step << " (body ";
           stmts(s->body);
@@ -924,6 +985,16 @@ void list_host(std::ostringstream& os, const Stmts& ss, int n) {
         os << ");\n";
         break;
       }
+      case Stmt::PersistentLaunch:
+        os << pad << "if (parpy_grid_fits_device(" << s->fname << ")) {   // all workgroups resident: the loop runs inside one kernel\n";
+        os << pad << "  " << s->fname << "<<<dim3(" << s->grid.x << ", " << s->grid.y << ", " << s->grid.z << "), dim3(" << s->block.x
+           << ", " << s->block.y << ", " << s->block.z << "), 0, 0>>>(";
+        for (size_t i = 0; i < s->args.size(); ++i) os << (i ? ", " : "") << print_expr(s->args[i]);
+        os << ", parpy_barrier_counter, parpy_barrier_status, parpy_barrier_limit);\n";
+        os << pad << "} else {\n";
+        list_host(os, s->body, n + 2);
+        os << pad << "}\n";
+        break;
       case Stmt::For:
         os << pad << "for (int64_t " << s->id.str() << " = " << print_expr(s->lo) << "; " << s->id.str() << (s->step > 0 ? " < " : " > ")
            << print_expr(s->hi) << "; " << s->id.str() << " += " << s->step << ") {\n";

@@ -72,6 +72,7 @@ Options parse_options(const std::string& sexpr) {
       }
     } else if (h == "debug_print") o.debug_print = flag();
     else if (h == "use_graphs") o.use_graphs = flag();
+    else if (h == "persistent_loops") o.persistent_loops = flag();
     else if (h == "force_int_size") { o.has_force_int = parse_elem_tag(f->at(1)->atom, &o.force_int); }
     else if (h == "force_float_size") { o.has_force_float = parse_elem_tag(f->at(1)->atom, &o.force_float); }
     else if (h == "includes") { for (size_t j = 1; j < f->size(); ++j) o.includes.push_back(f->at(j)->atom); }

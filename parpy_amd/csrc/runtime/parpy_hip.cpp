@@ -11,9 +11,11 @@
 #include <hip/hiprtc.h>
 
 #include <cmath>
+#include <cstdlib>
 #include <cstring>
 #include <map>
 #include <mutex>
+#include <set>
 #include <string>
 #include <vector>
 
@@ -78,7 +80,7 @@ struct HExpr {
 enum BinCode { ADD, SUB, MUL, DIV, FLOORDIV, REM, AND, OR, BITAND, BITOR, BITXOR, SHL, SHR, EQ, NEQ, LEQ, GEQ, LT, GT, MAX, MIN };
 
 struct HStmt {
-  enum Op : uint8_t { Launch, For, While, If, Def, Set, Alloc, Free } op = Launch;
+  enum Op : uint8_t { Launch, For, While, If, Def, Set, Alloc, Free, Persist } op = Launch;
   int kernel = -1;
   unsigned grid[3] = {1, 1, 1}, block[3] = {1, 1, 1};
   std::vector<HExpr> args;
@@ -86,7 +88,8 @@ struct HStmt {
   HExpr a, b;       // For: lo, hi; While/If: cond in a; Def/Set: value in a
   int64_t step = 1;
   int64_t nbytes = 0;
-  std::vector<HStmt> body, els;
+  std::vector<HStmt> body, els;   // Persist: body = the loop of launches that the kernel stands for
+  bool fits = false;              // Persist: every workgroup of the launch can be resident at once (checked at creation)
 };
 
 constexpr int64_t KEEP_LIMIT = int64_t(1) << 30;
@@ -158,7 +161,28 @@ struct Plan {
   int64_t scratch_top = 0;
   struct Carved { int slot; int64_t off; };
   std::vector<Carved> carved;
+  // Loops that run inside one kernel (persist statements): counter and status word of the device-wide
+  // barrier (32 bytes of device memory, allocated when the plan is created), whether a launch since the
+  // last check may have set the status, and how many runs used such a kernel.
+  unsigned* barrier_words = nullptr;
+  bool barrier_pending = false;
+  int64_t persistent_launches = 0;
 };
+
+// plans that own barrier words: parpy_sync looks at their status after the device has finished
+std::mutex g_plans_mu;
+std::set<Plan*> g_barrier_plans;
+
+int32_t check_barrier_status(Plan& p) {
+  if (!p.barrier_pending || !p.barrier_words) return 0;
+  p.barrier_pending = false;
+  unsigned status = 0;
+  if (int32_t rc = check(hipMemcpy(&status, p.barrier_words + 4, sizeof status, hipMemcpyDeviceToHost), "reading the barrier status")) return rc;
+  if (status != 0)
+    return fail("a barrier over all workgroups of a kernel that runs a whole loop of steps timed out: the workgroups "
+                "left the kernel early and its results are incomplete (PARPY_HIP_BARRIER_POLLS sets the limit)");
+  return 0;
+}
 
 struct PlanBuilder {
   Plan& p;
@@ -234,6 +258,34 @@ struct PlanBuilder {
       for (size_t k = 1; k < a->size(); ++k) s.args.push_back(expr(a->at(k)));
       if (s.args.size() != p.kparams[s.kernel].size())
         throw std::runtime_error("argument count mismatch for kernel " + p.knames[s.kernel]);
+    } else if (h == "persist") {
+      s.op = HStmt::Persist;
+      s.kernel = (int)x->at(1)->as_int();
+      if (s.kernel < 0 || s.kernel >= (int)p.fns.size()) throw std::runtime_error("launch of unknown kernel index");
+      for (int d = 0; d < 3; ++d) {
+        s.grid[d] = (unsigned)x->at(2 + d)->as_int();
+        s.block[d] = (unsigned)x->at(5 + d)->as_int();
+      }
+      const SXP& a = x->at(8);
+      for (size_t k = 1; k < a->size(); ++k) s.args.push_back(expr(a->at(k)));
+      // the kernel takes the barrier's counter, its status word and the poll limit after the plan's arguments
+      if (s.args.size() + 3 != p.kparams[s.kernel].size())
+        throw std::runtime_error("argument count mismatch for kernel " + p.knames[s.kernel]);
+      s.body = stmts(x->at(9), 1);
+      if (p.fns[s.kernel]) {
+        int per_cu = 0, cus = 0, dev = 0;
+        unsigned threads = s.block[0] * s.block[1] * s.block[2];
+        bool ok = hipGetDevice(&dev) == hipSuccess &&
+                  hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess &&
+                  hipModuleOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, p.fns[s.kernel], (int)threads, 0) == hipSuccess;
+        if (!ok) (void)hipGetLastError();
+        s.fits = ok && (int64_t)per_cu * cus >= (int64_t)s.grid[0] * s.grid[1] * s.grid[2];
+        if (s.fits && !p.barrier_words) {
+          void* w = nullptr;
+          if (hipMalloc(&w, 8 * sizeof(unsigned)) != hipSuccess) { (void)hipGetLastError(); s.fits = false; }
+          p.barrier_words = (unsigned*)w;
+        }
+      }
     } else if (h == "for") {
       s.op = HStmt::For;
       s.a = expr(x->at(2));
@@ -381,12 +433,16 @@ int32_t run_stmts(Plan& p, const std::vector<HStmt>& ss);
 
 int32_t run_stmt(Plan& p, const HStmt& s) {
   switch (s.op) {
-    case HStmt::Launch: {
+    case HStmt::Launch: case HStmt::Persist: {
+      const bool persist = s.op == HStmt::Persist;
+      // a loop inside one kernel needs its whole grid resident, memory for the barrier and a stream that is
+      // not being captured (the barrier words are cleared with a memset); otherwise the loop of launches runs
+      if (persist && !(s.fits && p.barrier_words && !p.capturing)) return run_stmts(p, s.body);
       const auto& kinds = p.kparams[s.kernel];
       Packed storage[64];
       void* ptrs[64];
       size_t n = s.args.size();
-      if (n > 64) return fail("kernel " + p.knames[s.kernel] + " has more than 64 parameters");
+      if (n + (persist ? 3 : 0) > 64) return fail("kernel " + p.knames[s.kernel] + " has more than 64 parameters");
       for (size_t k = 0; k < n; ++k) {
         Val v = eval(p, s.args[k]);
         Packed& q = storage[k];
@@ -406,6 +462,18 @@ int32_t run_stmt(Plan& p, const HStmt& s) {
           case Kind::F64: q.f64 = v.as_f(); break;
         }
         ptrs[k] = &storage[k];
+      }
+      if (persist) {
+        if (int32_t rc = check(hipMemsetAsync(p.barrier_words, 0, 8 * sizeof(unsigned), p.launch_stream), "clearing the barrier words")) return rc;
+        // polls of the counter before a workgroup gives up: about a microsecond each, two seconds by default
+        unsigned limit = 1u << 21;
+        if (const char* e = getenv("PARPY_HIP_BARRIER_POLLS")) limit = (unsigned)strtoul(e, nullptr, 10);
+        storage[n].p = p.barrier_words;
+        storage[n + 1].p = p.barrier_words + 4;   // 16 bytes on: both words are 16-byte aligned like every pointer argument
+        storage[n + 2].u32 = limit;
+        for (size_t k = n; k < n + 3; ++k) ptrs[k] = &storage[k];
+        p.barrier_pending = true;
+        ++p.persistent_launches;
       }
       ++p.launches;
       return check(hipModuleLaunchKernel(p.fns[s.kernel], s.grid[0], s.grid[1], s.grid[2], s.block[0], s.block[1],
@@ -513,7 +581,16 @@ void parpy_init(int64_t) {
   if (!scratch_on_current_device()) g_error = "no error";
 }
 
-int32_t parpy_sync(void) { return check(hipDeviceSynchronize(), "hipDeviceSynchronize"); }
+int32_t parpy_sync(void) {
+  if (int32_t rc = check(hipDeviceSynchronize(), "hipDeviceSynchronize")) return rc;
+  // kernels that run a loop of steps report a barrier that timed out through a status word
+  std::lock_guard<std::mutex> g(g_plans_mu);
+  for (Plan* p : g_barrier_plans) {
+    std::lock_guard<std::mutex> turn(p->mu);
+    if (int32_t rc = check_barrier_status(*p)) return rc;
+  }
+  return 0;
+}
 
 void* parpy_alloc_buffer(int64_t nbytes) {
   void* ptr = nullptr;
@@ -638,6 +715,10 @@ int32_t parpy_hip_plan_create(void* module, const char* plan_text, void** plan) 
     }
     p->body = b.stmts(x->at(4), 1);
     p->env.resize(p->slots.size());
+    if (p->barrier_words) {
+      std::lock_guard<std::mutex> g(g_plans_mu);
+      g_barrier_plans.insert(p);
+    }
   } catch (const std::exception& e) {
     delete p;
     return fail(std::string("invalid launch plan: ") + e.what());
@@ -752,6 +833,7 @@ int32_t parpy_hip_plan_run_timed(void* plan, void* const* args, int32_t nargs, f
   if (int32_t rc = plan_run_locked(p, args, nargs)) return rc;
   if (int32_t rc = check(hipEventRecord(p.ev_stop, nullptr), "hipEventRecord")) return rc;
   if (int32_t rc = check(hipEventSynchronize(p.ev_stop), "hipEventSynchronize")) return rc;
+  if (int32_t rc = check_barrier_status(p)) return rc;
   return check(hipEventElapsedTime(elapsed_ms, p.ev_start, p.ev_stop), "hipEventElapsedTime");
 }
 
@@ -780,8 +862,15 @@ int64_t parpy_hip_plan_launch_count(void* plan) { return ((Plan*)plan)->launches
 
 int64_t parpy_hip_plan_graph_replays(void* plan) { return ((Plan*)plan)->graph_replays; }
 
+int64_t parpy_hip_plan_persistent_launches(void* plan) { return ((Plan*)plan)->persistent_launches; }
+
 int32_t parpy_hip_plan_destroy(void* plan) {
   Plan* p = (Plan*)plan;
+  {
+    std::lock_guard<std::mutex> g(g_plans_mu);
+    g_barrier_plans.erase(p);
+  }
+  if (p->barrier_words) (void)hipFree(p->barrier_words);
   if (p->ev_start) (void)hipEventDestroy(p->ev_start);
   if (p->ev_stop) (void)hipEventDestroy(p->ev_stop);
   drop_graph(*p);

@@ -237,6 +237,7 @@ class CompileOptions:
         'use_cuda_thread_block_clusters': False,
         '_max_thread_blocks_per_cluster': 8,
         'use_cuda_graphs': False,
+        'persistent_loops': False,   # host loops of launches run inside one kernel with device-wide barriers when the grid fits
         '_force_int_size': None,
         '_force_float_size': None,
         'opt_vectorize': None,

@@ -75,6 +75,8 @@ def init_library(libpath):
     lib.parpy_hip_plan_set_graph.restype = i32
     lib.parpy_hip_plan_graph_replays.argtypes = [vp]
     lib.parpy_hip_plan_graph_replays.restype = i64
+    lib.parpy_hip_plan_persistent_launches.argtypes = [vp]
+    lib.parpy_hip_plan_persistent_launches.restype = i64
     lib.parpy_hip_plan_launch_count.argtypes = [vp]
     lib.parpy_hip_plan_launch_count.restype = i64
     lib.parpy_hip_plan_destroy.argtypes = [vp]

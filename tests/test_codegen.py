@@ -299,6 +299,23 @@ def o_for_alias():
     return opts_for({'N': parpy.threads(4), 'M': parpy.threads(64)}, opt_noalias_scopes=True)
 
 
+def test_persistent_loops_emit_one_kernel_for_the_host_loop_and_keep_the_loop_as_fallback():
+    hmm, seqs, args = _hmm_args(5)
+    o = opts_for({'inst': parpy.threads(4), 'state': parpy.threads(2048)}, persistent_loops=True)
+    s = compiles(parpy.print_compiled(W.forward_syn, args, o))
+    assert re.search(r"if \(parpy_grid_fits_device\(forward_syn_steps_\d+\)\)", s)
+    k = s[s.index("void __launch_bounds__(1024) forward_syn_steps_"):]
+    k = k[:k.index("\n}\n")]
+    assert re.search(r"for \(int t_\d+ = 1; t_\d+ < 30;", k) and "parpy_grid_barrier(" in k
+    # what the workgroups exchange is loaded and stored at device scope; the tables stay ordinary loads
+    assert "__hip_atomic_store(&alpha_dst" in k and "__hip_atomic_load(&alpha_src" in k
+    assert "__hip_atomic_load(&hmm_" not in k and "float* __restrict__ alpha" not in k
+    host = s[s.index("// host side"):]
+    assert re.search(r"\} else \{\n\s+for \(int64_t t_\d+ = 1; t_\d+ < 30;", host)
+    s0 = compiles(parpy.print_compiled(W.forward_syn, args, opts_for({'inst': parpy.threads(4), 'state': parpy.threads(2048)})))
+    assert "parpy_grid_fits_device" not in s0 and "_steps_" not in s0
+
+
 def test_hmm_multi_block_hoists_time_loop_to_host():
     hmm, seqs, args = _hmm_args(5, maxlen=20)
     s = compiles(parpy.print_compiled(W.forward_syn, args, opts_for({'inst': parpy.threads(4), 'state': parpy.threads(2048).tpb(512)})))

@@ -861,3 +861,59 @@ def test_forward_in_double_precision(k, threads):
     W.forward_syn(hd, sd, res, a1, a2, opts=opts_for({'inst': parpy.threads(n), 'state': parpy.threads(threads)}))
     want = oracle.hmm_syn_forward(hmm, seqs, np.float64)
     assert np.allclose(res.cpu().numpy(), want, atol=0, rtol=1e-12), np.abs(res.cpu().numpy() - want).max()
+
+
+# ---------------------------------------------------------------- loops of launches inside one kernel
+def test_persistent_step_loop_matches_the_loop_of_launches(golden_dir):
+    """`persistent_loops`: the host-hoisted time loop of the multi-block forward pass runs inside one kernel with a
+    barrier over all workgroups between steps (the grid of 2 x 100 workgroups is resident at once), same results."""
+    hmm, seqs, exp = _golden(golden_dir, 3)
+    hd, sd = W.to_device(hmm), W.to_device(seqs)
+    n, S = seqs["num_instances"], hmm["num_states"]
+    outs = []
+    for persistent in (False, True):
+        a1 = torch.zeros((n, S), dtype=torch.float32, device="cuda")
+        a2 = torch.zeros_like(a1)
+        res = torch.zeros(n, dtype=torch.float32, device="cuda")
+        o = opts_for({'inst': parpy.threads(n), 'state': parpy.threads(2048)}, persistent_loops=persistent)
+        W.forward_kernel(hd, sd, a1, a2, res, opts=o)
+        parpy.sync(HIP)
+        w = parpy._compile_function(parpy._ir_asts[W.forward_kernel], parpy.validate.check_arguments([hd, sd, a1, a2, res], o, True), o)
+        assert w.persistent_launches() == (1 if persistent else 0)
+        assert w.launch_count() < 20 if persistent else w.launch_count() > seqs["maxlen"] - 2
+        outs.append(res.cpu().numpy())
+    assert np.allclose(outs[1], exp, atol=1e-5, rtol=1e-5), np.abs(outs[1] - exp).max()
+    assert np.array_equal(outs[0], outs[1])
+
+
+def test_persistent_step_loop_on_the_synthetic_model_and_fallback_when_the_grid_does_not_fit():
+    hmm, seqs = W.synthetic_hmm(5, n_inst=6, min_len=20, max_len=120)
+    want = oracle.hmm_syn_forward(hmm, seqs, np.float32)
+    got, _, _ = _run_synthetic(hmm, seqs, 4096, persistent_loops=True)          # 4 workgroups per read
+    assert np.allclose(got, want, atol=1e-5, rtol=1e-5), np.abs(got - want).max()
+    # 600 reads x 4 workgroups of 1024 threads cannot all be resident: the loop of launches runs instead
+    hmm, seqs = W.synthetic_hmm(5, n_inst=600, min_len=5, max_len=12)
+    want = oracle.hmm_syn_forward(hmm, seqs, np.float32)
+    got, _, _ = _run_synthetic(hmm, seqs, 4096, persistent_loops=True)
+    assert np.allclose(got, want, atol=1e-5, rtol=1e-5), np.abs(got - want).max()
+
+
+def test_persistent_step_loop_reports_a_barrier_that_times_out(monkeypatch):
+    """With a poll limit of zero the first workgroup that has to wait gives up: every workgroup leaves the kernel
+    (it ends normally) and the next synchronisation raises."""
+    hmm, seqs = W.synthetic_hmm(5, n_inst=6, min_len=300, max_len=400)
+    hd, sd = W.to_device(hmm), W.to_device(seqs)
+    n, S = seqs["num_instances"], hmm["num_states"]
+    a1 = torch.zeros((n, S), dtype=torch.float32, device="cuda")
+    a2 = torch.zeros_like(a1)
+    res = torch.zeros(n, dtype=torch.float32, device="cuda")
+    o = opts_for({'inst': parpy.threads(n), 'state': parpy.threads(4096)}, persistent_loops=True)
+    monkeypatch.setenv("PARPY_HIP_BARRIER_POLLS", "0")
+    W.forward_syn(hd, sd, res, a1, a2, opts=o)
+    with pytest.raises(RuntimeError, match="barrier over all workgroups .* timed out"):
+        parpy.sync(HIP)
+    monkeypatch.delenv("PARPY_HIP_BARRIER_POLLS")
+    W.forward_syn(hd, sd, res, a1, a2, opts=o)
+    parpy.sync(HIP)
+    want = oracle.hmm_syn_forward(hmm, seqs, np.float32)
+    assert np.allclose(res.cpu().numpy(), want, atol=1e-5, rtol=1e-5)
