@@ -398,7 +398,7 @@ struct Inliner {
     if (f.params.size() != r->args.size())
       fail_rt(r->i, "Function " + f.id.s + " expected " + std::to_string(f.params.size()) + " arguments, but received " +
                         std::to_string(r->args.size()) + ".");
-    if (f.body.empty() || f.body.back()->k != Stmt::Return)
+    if (f.body.empty() || !always_returns(f.body))
       fail_ty(r->i, "Unknown return type of function " + f.id.s);
     Sub sub;
     for (size_t k = 0; k < f.params.size(); ++k) {
@@ -415,9 +415,72 @@ struct Inliner {
       }
       sub.params[f.params[k].id] = a;
     }
-    Stmts head(f.body.begin(), f.body.end() - 1);
-    for (auto& st : sub_stmts(head, sub)) pre.push_back(st);
-    return sub_expr(f.body.back()->expr, sub);
+    if (count_returns(f.body) == 1 && f.body.back()->k == Stmt::Return) {
+      Stmts head(f.body.begin(), f.body.end() - 1);
+      for (auto& st : sub_stmts(head, sub)) pre.push_back(st);
+      return sub_expr(f.body.back()->expr, sub);
+    }
+    // Several return statements (`if c: return a` ... `return b`).  The reference keeps such a callee as a device
+    // function (src/py/insert_called_functions.rs:12-88); here the body is inlined like any other with the
+    // returned value in a variable: what follows a conditional that returns moves into the branch that goes on,
+    // every `return e` becomes `result = e`.  The variable takes the type of the first value assigned to it.
+    if (return_in_loop(f.body, false))
+      fail_rt(r->i, "A return statement inside a loop of function " + f.id.s + " is not supported when the call is part of an expression");
+    Name res = gen.fresh(f.id.s + "_result");
+    E resv = mk_var(res, Type(), r->i);
+    auto marker = std::make_shared<Expr>();
+    marker->k = Expr::NeutralElement;   // without operand: a definition whose type comes from the first assignment
+    marker->bop = BinOp::Add;
+    marker->i = r->i;
+    pre.push_back(mk_def(res, Type(), marker, r->i));
+    for (auto& st : sub_stmts(lower_returns(f.body, resv), sub)) pre.push_back(st);
+    return resv;
+  }
+
+  static int count_returns(const Stmts& ss) {
+    int n = 0;
+    for (auto& s : ss) n += (s->k == Stmt::Return) + count_returns(s->body) + count_returns(s->els);
+    return n;
+  }
+
+  static bool return_in_loop(const Stmts& ss, bool in_loop) {
+    for (auto& s : ss) {
+      if (s->k == Stmt::Return && in_loop) return true;
+      bool loop = in_loop || s->k == Stmt::For || s->k == Stmt::While;
+      if (return_in_loop(s->body, loop) || return_in_loop(s->els, loop)) return true;
+    }
+    return false;
+  }
+
+  static bool always_returns(const Stmts& ss) {
+    if (ss.empty()) return false;
+    const S& last = ss.back();
+    if (last->k == Stmt::Return) return true;
+    return last->k == Stmt::If && always_returns(last->body) && always_returns(last->els);
+  }
+
+  static Stmts lower_returns(const Stmts& ss, const E& res) {
+    Stmts out;
+    for (size_t i = 0; i < ss.size(); ++i) {
+      const S& s = ss[i];
+      if (s->k == Stmt::Return) {
+        out.push_back(mk_assign(res, s->expr, s->i));
+        return out;   // nothing after a return runs
+      }
+      if (s->k == Stmt::If && (count_returns(s->body) || count_returns(s->els))) {
+        Stmts rest(ss.begin() + i + 1, ss.end());
+        Stmts b = s->body, e = s->els;
+        if (!always_returns(b)) b.insert(b.end(), rest.begin(), rest.end());
+        if (!always_returns(e)) e.insert(e.end(), rest.begin(), rest.end());
+        auto r = std::make_shared<Stmt>(*s);
+        r->body = lower_returns(b, res);
+        r->els = lower_returns(e, res);
+        out.push_back(r);
+        return out;
+      }
+      out.push_back(s);
+    }
+    return out;
   }
 
   Stmts sub_stmts(const Stmts& ss, Sub& sub) {

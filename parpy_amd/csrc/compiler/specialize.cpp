@@ -638,8 +638,28 @@ struct TypeChecker {
   const Options& opts;
   std::map<Name, Type> vars;
   Type res_ty = Type::vvoid();
+  std::set<Name> pending;             // result variables of inlined calls that have not been assigned yet
+  std::map<Name, Type> resolved;      // ... and the type their first assignment gave them
 
   explicit TypeChecker(const Options& o) : opts(o) {}
+
+  // definitions left without a value get the zero of the type they were resolved to
+  Stmts finish(const Stmts& ss) {
+    Stmts out;
+    for (auto& s : ss) {
+      auto r = std::make_shared<Stmt>(*s);
+      if (s->k == Stmt::Def && s->expr->k == Expr::NeutralElement && s->expr->args.empty()) {
+        auto it = resolved.find(s->id);
+        if (it == resolved.end()) fail_ty(s->i, "Unknown return type of a called function (no value is ever returned)");
+        r->ty = it->second;
+        r->expr = is_float(r->ty.sz) ? mk_float(0.0, r->ty.sz, s->i) : r->ty.sz == ElemSize::Bool ? mk_bool(false, s->i) : mk_int(0, r->ty.sz, s->i);
+      }
+      r->body = finish(s->body);
+      r->els = finish(s->els);
+      out.push_back(r);
+    }
+    return out;
+  }
 
   static bool is_scalar_of(const Type& t, bool (*pred)(ElemSize)) { return t.is_scalar() && pred(t.sz); }
 
@@ -924,6 +944,11 @@ struct TypeChecker {
     auto r = std::make_shared<Stmt>(*s);
     switch (s->k) {
       case Stmt::Def: {
+        if (s->expr->k == Expr::NeutralElement && s->expr->args.empty()) {
+          // the result variable of an inlined call with several returns: typed by its first assignment
+          pending.insert(s->id);
+          break;
+        }
         r->expr = expr(s->expr);
         r->ty = r->expr->ty;
         if (r->ty.k != Type::Tensor) fail_ty(s->i, "Unsupported type " + r->ty.str() + " of variable " + s->id.s);
@@ -931,6 +956,15 @@ struct TypeChecker {
         break;
       }
       case Stmt::Assign: {
+        if (s->dst->k == Expr::Var && pending.count(s->dst->name)) {
+          r->expr = expr(s->expr);
+          if (!r->expr->ty.is_scalar()) fail_ty(s->i, "Unsupported type " + r->expr->ty.str() + " of the value returned by a called function");
+          vars[s->dst->name] = r->expr->ty;
+          resolved[s->dst->name] = r->expr->ty;
+          pending.erase(s->dst->name);
+          r->dst = with_type(s->dst, r->expr->ty);
+          break;
+        }
         r->dst = expr(s->dst);
         r->expr = coerce(expr(s->expr), r->dst->ty);
         break;
@@ -1015,7 +1049,7 @@ FunDef specialize(const ParsedFun& pf, const std::vector<ArgDesc>& args, const O
 
   TypeChecker tc(opts);
   for (auto& p : out.params) tc.vars[p.id] = p.ty;
-  body = tc.stmts(body);
+  body = tc.finish(tc.stmts(body));
   out.body = fold_stmts(body);
   return out;
 }

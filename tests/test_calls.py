@@ -150,6 +150,48 @@ def sum_rows_using_ext(out, x, N):
         out[i] = wave_sum_custom(x[i])
 
 
+# callees with more than one return statement (the reference keeps them as device functions,
+# src/py/insert_called_functions.rs:12-88; here they are inlined with the returned value in a variable)
+@parpy.jit
+def clamp_between(x, lo, hi):
+    if x < lo:
+        return lo
+    if x > hi:
+        return hi
+    return x
+
+
+@parpy.jit
+def piecewise(x, y):
+    t = x * y
+    if t > 1.0:
+        u = t - 1.0
+        return u * u
+    elif t < -1.0:
+        return -t
+    v = t + 2.0
+    return v
+
+
+@parpy.jit
+def sign_of(x):
+    if x > 0.0:
+        return 1
+    else:
+        if x < 0.0:
+            return -1
+        else:
+            return 0
+
+
+@parpy.jit
+def early_returns(x, y, sgn, N):
+    parpy.label('N')
+    for i in range(N):
+        y[i] = clamp_between(x[i], parpy.operators.float32(-1.0), parpy.operators.float32(2.0)) + piecewise(x[i], y[i])
+        sgn[i] = sign_of(x[i])
+
+
 F = np.float32
 
 
@@ -160,6 +202,36 @@ def test_expression_calls_are_inlined():
     assert "add_call" not in s.split("extern \"C\" __global__")[1]
     compiles(parpy.print_compiled(add_mul_nested, [x, x.copy(), 10], opts_for({'N': parpy.threads(10)})))
     compiles(parpy.print_compiled(with_locals, [x, x.copy(), 10], opts_for({'N': parpy.threads(10)})))
+
+
+def test_callees_with_several_returns_are_inlined_through_a_result_variable():
+    x = np.zeros(10, dtype=F)
+    s = compiles(parpy.print_compiled(early_returns, [x, x.copy(), np.zeros(10, dtype=np.int64), 10], opts_for({'N': parpy.threads(10)})))
+    assert re.search(r"float clamp_between_result_\d+ = 0.0f;", s) and re.search(r"int64_t sign_of_result_\d+ = 0;", s)
+    with pytest.raises(RuntimeError, match="return statement inside a loop"):
+        @parpy.jit
+        def first_positive(x: types.F32):
+            for k in range(3):
+                if x > k:
+                    return k
+            return 3
+
+        @parpy.jit
+        def use(x, y, N):
+            parpy.label('N')
+            for i in range(N):
+                y[i] = first_positive(x[i])
+    with pytest.raises(TypeError, match="Unknown return type"):
+        @parpy.jit
+        def maybe(x: types.F32):
+            if x > 0.0:
+                return x
+
+        @parpy.jit
+        def use2(x, y, N):
+            parpy.label('N')
+            for i in range(N):
+                y[i] = maybe(x[i])
 
 
 def test_statement_calls_with_sub_tensors():
@@ -273,6 +345,20 @@ def test_calls_give_the_results_of_the_inlined_code():
     a3, b3 = rng.standard_normal((10, 20, 30)).astype(F), np.zeros((10, 20, 30), dtype=F)
     add_3d_inplace(a3, b3, 10, 20, 30, opts=opts_for({'3d': parpy.threads(10), '2d': parpy.threads(20), '1d': parpy.threads(30)}))
     assert np.array_equal(a3, b3)
+
+
+@pytest.mark.gpu
+def test_callees_with_several_returns_give_what_python_gives():
+    rng = np.random.default_rng(13)
+    x = (3.0 * rng.standard_normal(500)).astype(F)
+    y0 = rng.standard_normal(500).astype(F)
+    y, sgn = y0.copy(), np.zeros(500, dtype=np.int64)
+    early_returns(x, y, sgn, 500, opts=opts_for({'N': parpy.threads(500)}))
+    t = x.astype(np.float64) * y0
+    pw = np.where(t > 1.0, (t - 1.0) ** 2, np.where(t < -1.0, -t, t + 2.0))
+    want = np.clip(x, -1.0, 2.0) + pw
+    assert np.allclose(y, want, rtol=1e-6, atol=1e-6)
+    assert np.array_equal(sgn, np.sign(x).astype(np.int64))
 
 
 @pytest.mark.gpu
