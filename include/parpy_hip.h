@@ -18,8 +18,12 @@
  *
  * All work is enqueued on the null stream and is not synchronised before
  * returning (like the reference).  No torch or Python types appear here.
- * Thread-safety: none promised beyond what HIP gives; the error message is a
- * per-thread buffer owned by the library.
+ * Threads: the error message is a per-thread buffer owned by the library;
+ * runs of one launch plan from several host threads take turns, different
+ * plans run side by side; nothing else is promised beyond what HIP gives.
+ * Host-side integer expressions of a plan are evaluated in signed 64-bit
+ * arithmetic (unsigned 64-bit values above 2^63 are not represented); a
+ * division by zero there fails the run with a message.
  */
 #ifndef PARPY_HIP_H
 #define PARPY_HIP_H
@@ -72,7 +76,10 @@ int32_t parpy_hip_plan_create(void* module, const char* plan_text, void** plan);
  * folded into the code at compile time.  Returns 0 or non-zero.  A plan holds
  * the state of its host loops and its device temporaries: runs of one plan
  * from several host threads take turns (different plans run concurrently);
- * the error message is per thread. */
+ * the error message is per thread.  Temporaries stay allocated between runs up
+ * to 1 GiB per plan and 8 GiB over all plans of the process (beyond that they
+ * are allocated and freed per run); a run that fails half way frees what it
+ * had allocated for itself. */
 int32_t parpy_hip_plan_run(void* plan, void* const* args, int32_t nargs);
 
 /* Same as parpy_hip_plan_run, bracketed by HIP events recorded on the null

@@ -10,6 +10,7 @@
 #include <hip/hip_runtime.h>
 #include <hip/hiprtc.h>
 
+#include <atomic>
 #include <cmath>
 #include <cstdlib>
 #include <cstring>
@@ -92,7 +93,10 @@ struct HStmt {
   bool fits = false;              // Persist: every workgroup of the launch can be resident at once (checked at creation)
 };
 
-constexpr int64_t KEEP_LIMIT = int64_t(1) << 30;
+constexpr int64_t KEEP_LIMIT = int64_t(1) << 30;         // per plan
+constexpr int64_t KEEP_LIMIT_ALL = int64_t(8) << 30;     // over all live plans of the process
+std::atomic<int64_t> g_kept_all{0};
+thread_local bool g_div_by_zero = false;                  // set by eval, checked after every statement
 
 }  // namespace
 
@@ -137,6 +141,7 @@ struct Plan {
   struct Kept { void* ptr = nullptr; int64_t nbytes = 0; bool in_use = false; };
   std::vector<Kept> kept;
   int64_t kept_bytes = 0;
+  std::vector<void*> unkept;   // temporaries of the current run that are freed when it ends, also when it fails half way
   hipEvent_t ev_start = nullptr, ev_stop = nullptr;  // created on the first timed run
   // Graph replay (the analogue of the reference's use_cuda_graphs, src/cuda/graphs.rs): the
   // launches of one run are captured into a HIP graph and later runs with the same pointer
@@ -389,8 +394,8 @@ Val eval(const Plan& p, const HExpr& e) {
         case ADD: r.i = x + y; break;
         case SUB: r.i = x - y; break;
         case MUL: r.i = x * y; break;
-        case DIV: case FLOORDIV: r.i = y ? x / y : 0; break;
-        case REM: r.i = y ? x % y : 0; break;
+        case DIV: case FLOORDIV: if (y == 0) g_div_by_zero = true; r.i = y ? x / y : 0; break;
+        case REM: if (y == 0) g_div_by_zero = true; r.i = y ? x % y : 0; break;
         case AND: r.i = (x != 0) && (y != 0); break;
         case OR: r.i = (x != 0) || (y != 0); break;
         case BITAND: r.i = x & y; break;
@@ -529,11 +534,14 @@ int32_t run_stmt(Plan& p, const HStmt& s) {
       if (int32_t rc = check(e, "allocation of a device temporary")) return rc;
       p.env[s.slot].t = Val::P;
       p.env[s.slot].p = ptr;
-      if (!kp.ptr && p.kept_bytes + s.nbytes <= KEEP_LIMIT) {
+      if (!kp.ptr && p.kept_bytes + s.nbytes <= KEEP_LIMIT && g_kept_all.load() + s.nbytes <= KEEP_LIMIT_ALL) {
         kp.ptr = ptr;
         kp.nbytes = s.nbytes;
         kp.in_use = true;
         p.kept_bytes += s.nbytes;
+        g_kept_all += s.nbytes;
+      } else {
+        p.unkept.push_back(ptr);
       }
       return 0;
     }
@@ -553,6 +561,8 @@ int32_t run_stmt(Plan& p, const HStmt& s) {
         p.kept[s.slot].in_use = false;  // stays allocated for the next run
         return 0;
       }
+      for (size_t k = 0; k < p.unkept.size(); ++k)
+        if (p.unkept[k] == ptr) { p.unkept.erase(p.unkept.begin() + k); break; }
       hipError_t e = hipFreeAsync(ptr, nullptr);
       if (e != hipSuccess) {
         (void)hipGetLastError();
@@ -565,9 +575,21 @@ int32_t run_stmt(Plan& p, const HStmt& s) {
 }
 
 int32_t run_stmts(Plan& p, const std::vector<HStmt>& ss) {
-  for (auto& s : ss)
+  for (auto& s : ss) {
     if (int32_t rc = run_stmt(p, s)) return rc;
+    if (g_div_by_zero) return fail("division by zero in the host part of the launch plan");
+  }
   return 0;
+}
+
+// what a run that stopped half way still holds
+void release_unkept(Plan& p) {
+  for (void* ptr : p.unkept)
+    if (hipFreeAsync(ptr, nullptr) != hipSuccess) {
+      (void)hipGetLastError();
+      (void)hipFree(ptr);
+    }
+  p.unkept.clear();
 }
 
 }  // namespace
@@ -807,7 +829,13 @@ int32_t plan_run_locked(Plan& p, void* const* args, int32_t nargs) {
     for (auto& kp : p.kept) kp.in_use = false;
   }
   p.launches = 0;
+  g_div_by_zero = false;
   int32_t rc = run_stmts(p, p.body);
+  if (rc != 0) {
+    std::string msg = g_error;
+    release_unkept(p);
+    g_error = msg;
+  }
   if (p.use_graph && p.graph_state == 0) p.graph_state = rc == 0 ? 1 : -1;  // temporaries exist now: capture from the next run on
   return rc;
 }
@@ -853,6 +881,7 @@ int32_t parpy_hip_plan_run_noalloc(void* plan, void* const* args, int32_t nargs)
   p.scratch_top = 0;
   p.carved.clear();
   p.launches = 0;
+  g_div_by_zero = false;
   int32_t rc = run_stmts(p, p.body);   // eager launches on the null stream; no graph, no kept temporaries
   p.scratch_base = nullptr;
   return rc;
@@ -877,6 +906,7 @@ int32_t parpy_hip_plan_destroy(void* plan) {
   if (p->cap_stream) (void)hipStreamDestroy(p->cap_stream);
   for (auto& kp : p->kept)
     if (kp.ptr) (void)hipFree(kp.ptr);
+  g_kept_all -= p->kept_bytes;
   delete p;
   return 0;
 }

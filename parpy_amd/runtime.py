@@ -22,7 +22,8 @@ libs = {}
 
 
 def build_library(force=False):
-    """Compile csrc/runtime/parpy_hip.cpp with hipcc (host code only; cross-compiles without a GPU)."""
+    """Compile csrc/runtime/parpy_hip.cpp with hipcc for gfx950 (host code plus the device scratch array;
+    cross-compiles without a GPU)."""
     src = PARPY_NATIVE_PATH / "parpy_hip.cpp"
     deps = [src, pathlib.Path(__file__).parent / "csrc" / "compiler" / "sexpr.hpp",
             pathlib.Path(__file__).parent.parent / "include" / "parpy_hip.h"]

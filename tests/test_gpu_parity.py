@@ -560,6 +560,22 @@ def test_compile_string_and_runtime_error_paths():
     lib = _compile_runtime_lib(HIP)
     assert not lib.parpy_alloc_buffer(1 << 60)                      # absurd allocation: NULL and a message
     assert len(lib.parpy_get_error_message()) > 0
+    # a plan whose host part divides by zero fails the run instead of carrying on with 0; the temporary that the
+    # run had allocated for itself (too large to be kept between runs) is released on the way out
+    import ctypes
+    from parpy_amd.compile import _modules
+    module = list(_modules.values())[-1][0]
+    text = (b'(plan "f" (params ("x" ptr)) (kernels) (body (alloc "big" 2147483648) '
+            b'(def "a" i64 (bin floordiv i (i 1) (i 0))) (free "big")))')
+    plan = ctypes.c_void_p()
+    assert lib.parpy_hip_plan_create(module, text, ctypes.byref(plan)) == 0
+    args = (ctypes.c_void_p * 1)(x.data_ptr())
+    free_before = torch.cuda.mem_get_info()[0]
+    assert lib.parpy_hip_plan_run(plan, args, 1) != 0
+    assert b"division by zero" in lib.parpy_get_error_message()
+    parpy.sync(HIP)
+    assert torch.cuda.mem_get_info()[0] >= free_before - (64 << 20)
+    assert lib.parpy_hip_plan_destroy(plan) == 0
 
 
 def test_timed_call_and_launch_count():
