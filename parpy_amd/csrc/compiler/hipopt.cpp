@@ -508,6 +508,160 @@ struct Pass {
     return out;
   }
 
+  // ================================================================ rows selected by a value loaded one step ahead
+  // Second level of the step-ahead loads above: `o = o_next; o_next = data[i, t + 1]` makes the observation of
+  // the next step known while the current one runs, so the elements of a never-written table that a thread
+  // reads at `tab[o, f(iteration)]` can be fetched for step t + 1 as soon as the thread has consumed those of
+  // step t.  They travel in a per-thread register array (one slot per iteration the thread runs): filled
+  // before the loop for the first step, refilled right after the thread's loop over its iterations, so the
+  // latency of the table passes behind the barrier and the shared-memory phase of the next step.  Costs one
+  // register per element and is only done while the register budget lasts.
+  Stmts prefetch_selected_rows(const Stmts& ss, int64_t* budget) {
+    std::set<Name> params = param_names();
+    std::set<Name> written = written_arrays();
+    Stmts out;
+    for (auto& s : ss) {
+      bool seq = s->k == Stmt::For && s->map.k == GpuMap::None && !s->unroll;
+      // the pairs `o = o_next; o_next = ...` at the top level of the loop body
+      std::map<Name, Name> ahead;   // o -> o_next
+      if (seq)
+        for (size_t i = 0; i + 1 < s->body.size(); ++i) {
+          const S &d = s->body[i], &a = s->body[i + 1];
+          if (d->k == Stmt::Def && d->expr && d->expr->k == Expr::Var && a->k == Stmt::Assign && a->dst->k == Expr::Var &&
+              a->dst->name == d->expr->name && has_load(a->expr))
+            ahead[d->id] = d->expr->name;
+        }
+      if (!seq || ahead.empty()) {
+        auto r = clone(s);
+        r->body = prefetch_selected_rows(s->body, budget);
+        r->els = prefetch_selected_rows(s->els, budget);
+        out.push_back(r);
+        continue;
+      }
+      std::set<Name> varying;
+      visit_stmts(s->body, [&](const S& c) {
+        if (c->k == Stmt::Def || c->k == Stmt::For) varying.insert(c->id);
+        if (c->k == Stmt::Assign && c->dst->k == Expr::Var) varying.insert(c->dst->name);
+      });
+      Stmts pre, body;
+      for (auto& c : s->body) {
+        IterSpace is;
+        if (!(thread_mapped(c) && iter_space(c, &is))) { body.push_back(c); continue; }
+        std::set<Name> iter_vars{c->id};
+        if (is.inner) iter_vars.insert(is.inner->id);
+        std::map<Name, E> defs;   // definitions in the body that are pure functions of the iteration
+        std::function<void(const Stmts&)> collect_defs = [&](const Stmts& b) {
+          for (auto& d : b) {
+            if (d->k == Stmt::Def && d->ty.is_scalar() && !has_load(d->expr)) {
+              E e = subst_vars(d->expr, defs);
+              bool pure = true;
+              visit_exprs(e, [&](const E& x) { if (x->k == Expr::Var && !iter_vars.count(x->name)) pure = false; });
+              if (pure) defs[d->id] = e;
+            }
+            collect_defs(d->body);
+            collect_defs(d->els);
+          }
+        };
+        collect_defs(*is.body);
+        struct Row { E load; Name reg; ElemSize sz; };
+        std::vector<Row> rows;
+        auto take = [&](const E& e) -> E {
+          if (e->k != Expr::Index || e->args[0]->k != Expr::Var) return e;
+          const Name& base = e->args[0]->name;
+          if (!params.count(base) || written.count(base) || e->dim_shape.empty() || elem_bytes(e->ty.sz) > 4) return e;
+          E idx = fold_expr(subst_vars(e->args[1], defs));
+          bool selected = false, ok = true;
+          visit_exprs(idx, [&](const E& x) {
+            if (x->k == Expr::Var && ahead.count(x->name)) selected = true;
+            else if (x->k == Expr::Var && !iter_vars.count(x->name) && varying.count(x->name)) ok = false;
+            if (x->k == Expr::Index || x->k == Expr::RegElem || x->k == Expr::ThreadIdx || x->k == Expr::Call || x->k == Expr::Raw) ok = false;
+          });
+          if (!selected || !ok) return e;
+          auto elem = [&](const Name& reg) {
+            auto re = std::make_shared<Expr>();
+            re->k = Expr::RegElem;
+            re->ty = e->ty;
+            re->name = reg;
+            re->args = {is.slot};
+            return E(re);
+          };
+          for (auto& r : rows)
+            if (r.load->args[0]->name == base && expr_eq(r.load->args[1], idx)) return elem(r.reg);
+          auto ld = std::make_shared<Expr>(*e);
+          ld->args = {e->args[0], idx};
+          ld->dim_idx.clear();
+          rows.push_back({E(ld), gen.fresh("row_" + base.s), e->ty.sz});
+          return elem(rows.back().reg);
+        };
+        Stmts nbody = rewrite_stmts(*is.body, take);
+        // all elements of the row that the thread reads, or none (a part of them would split the 16-byte loads)
+        int64_t cost = (int64_t)rows.size() * is.slots;
+        if (rows.empty() || *budget < cost) { body.push_back(c); continue; }
+        *budget -= cost;
+        // the loop nest that fills the registers from the row of the step to come
+        auto fill_nest = [&]() {
+          std::map<Name, E> rv;
+          Type ity = Type::scalar(isz);
+          Name nq = gen.fresh(c->id.s), nu;
+          rv[c->id] = mk_var(nq, ity);
+          if (is.inner) { nu = gen.fresh(is.inner->id.s); rv[is.inner->id] = mk_var(nu, ity); }
+          for (auto& kv : ahead) rv[kv.first] = mk_var(kv.second, Type::scalar(ElemSize::I8));
+          auto outer = clone(c);
+          outer->id = nq;
+          outer->unroll = true;
+          E kq = counter_var(outer, isz), slot = kq;
+          if (is.inner) {
+            int64_t V = const_extent(is.inner);
+            slot = fold_expr(mk_binop(BinOp::Add, mk_binop(BinOp::Mul, kq, mk_int(V, isz), ity), mk_var(nu, ity), ity));
+          }
+          Stmts fills;
+          for (auto& r : rows) {
+            auto re = std::make_shared<Expr>();
+            re->k = Expr::RegElem;
+            re->ty = Type::scalar(r.sz);
+            re->name = r.reg;
+            re->args = {slot};
+            fills.push_back(mk_assign(E(re), subst_vars(r.load, rv)));
+          }
+          if (is.inner) {
+            auto fi = clone(is.inner);
+            fi->id = nu;
+            fi->body = fills;
+            outer->body = {S(fi)};
+          } else {
+            outer->body = fills;
+          }
+          return S(outer);
+        };
+        for (auto& r : rows) {
+          auto d = std::make_shared<Stmt>();
+          d->k = Stmt::RegDecl;
+          d->id = r.reg;
+          d->ty = Type::scalar(r.sz);
+          d->iv = is.slots;
+          pre.push_back(d);
+        }
+        pre.push_back(fill_nest());
+        auto nc = clone(c);
+        nc->unroll = true;
+        if (is.inner) {
+          auto ni = clone(is.inner);
+          ni->body = nbody;
+          nc->body = {S(ni)};
+        } else {
+          nc->body = nbody;
+        }
+        body.push_back(nc);
+        body.push_back(fill_nest());
+      }
+      for (auto& d : pre) out.push_back(d);
+      auto r = clone(s);
+      r->body = body;
+      out.push_back(r);
+    }
+    return out;
+  }
+
   // ================================================================ conditions no iteration changes
   // A parallel loop whose whole body is `if (c) A else B`, with c the same for every iteration (it
   // mentions neither the loop variable nor anything the body defines or assigns, and loads only from
@@ -1075,7 +1229,28 @@ struct Pass {
     int64_t threads = k.block.x * k.block.y * k.block.z;
     // a 1024-thread block leaves 128 VGPRs per lane; 88 cached values plus the
     // working set fit without spilling (measured on the HMM kernels; 96 spills a few)
-    return threads <= 256 ? 192 : threads <= 512 ? 128 : 88;
+    if (threads <= 512) return threads <= 256 ? 192 : 128;
+    // a per-element step body without exponentials or logarithms keeps few values alive besides the cached ones
+    bool transcendental = false;
+    std::function<void(const Stmts&, bool, bool)> walk = [&](const Stmts& ss, bool in_seq, bool in_threads) {
+      for (auto& st : ss) {
+        if (in_seq && in_threads) {
+          auto scan = [&](const E& e) {
+            visit_exprs(e, [&](const E& x) { if (x->k == Expr::UnOpE && (x->uop == UnOp::Exp || x->uop == UnOp::Log)) transcendental = true; });
+          };
+          scan(st->expr);
+          scan(st->dst);
+        }
+        bool seq = st->k == Stmt::For && st->map.k == GpuMap::None && !st->unroll;
+        bool thr = st->k == Stmt::For && st->map.k == GpuMap::Thread;
+        // (reductions of a whole row every few steps are not the step body: only straight element loops count)
+        bool reduction_like = thr && st->par.reduction;
+        walk(st->body, in_seq || seq, in_threads || (thr && !reduction_like));
+        walk(st->els, in_seq, in_threads);
+      }
+    };
+    walk(k.body, false, false);
+    return transcendental ? 88 : 104;
   }
 
   // hoist out of the sequential loop `seq` (a statement of `parent`)
@@ -2501,6 +2676,7 @@ void hip_optimize(Program& p, const Options& opts, NameGen& gen) {
     if (opts.opt_vectorize) k.body = pass.vectorize(k.body);
     int64_t budget = pass.reg_budget();
     if (opts.opt_hoist_invariant) k.body = pass.hoist_invariant(k.body, &budget, false);
+    if (opts.opt_prefetch_steps) k.body = pass.prefetch_selected_rows(k.body, &budget);
     if (opts.opt_reg_cache) pass.reg_cache(&budget);
     if (opts.opt_drop_barriers) pass.drop_barriers();
     if (opts.opt_noalias_scopes) k.body = pass.noalias_scopes(k.body);

@@ -201,6 +201,7 @@ __device__ __forceinline__ bool parpy_grid_barrier(unsigned* counter, unsigned* 
   return parpy_bar_ok != 0;
 }
 typedef float parpy_f32x4 __attribute__((ext_vector_type(4)));
+template <class T> using parpy_vec4 = T __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ int parpy_lane_id() { return (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)); }
 // dst[c][r] = src[r][c] for a ROWS x COLS matrix in 64 x 64 tiles: a 256-thread workgroup reads
 // 64-word row segments of its tile, turns the tile round in LDS and writes 64-word row segments
@@ -468,6 +469,10 @@ struct DevicePrinter {
       case Expr::IfExpr: return "(" + pexpr(e->args[0]) + " ? " + pexpr(e->args[1]) + " : " + pexpr(e->args[2]) + ")";
       case Expr::Convert: return "((" + std::string(elem_ctype(e->ty.sz)) + ")" + paren(pexpr(e->args[0])) + ")";
       case Expr::Index: {
+        if (!as_lvalue) {
+          auto pk = pack_loads.find(e.get());
+          if (pk != pack_loads.end()) return pk->second;
+        }
         // Indexing is in bounds by contract: a variable used as the index of one dimension lies in
         // [0, extent) while this address is computed, which lets gathered indices (loaded from memory,
         // so of unknown range) take part in 32-bit address arithmetic.
@@ -720,6 +725,13 @@ struct DevicePrinter {
       case Stmt::Assign: {
         std::string rhs = pexpr(s->expr);
         if (s->dst->k == Expr::Var && !s->dst->ty.is_scalar()) rhs = "(" + ctype(s->dst->ty) + ")" + rhs;
+        {
+          auto pk = pack_stores.find(s.get());
+          if (pk != pack_stores.end()) {
+            os << ind(n) << packs[pk->second.first].var << "." << "xyzw"[pk->second.second] << " = " << rhs << ";\n";
+            break;
+          }
+        }
         if (s->dst->k == Expr::Index && s->dst->args[0]->k == Expr::Var && stream_out.count(s->dst->args[0]->name) &&
             elem_bytes(s->dst->ty.sz) >= 4) {
           // write-once data bypasses the caches on its way to HBM (measured: 7.1 instead of 5.8 TB/s on a plain copy)
@@ -800,8 +812,189 @@ struct DevicePrinter {
     }
   }
 
+  // ---- four adjacent 4-byte accesses of one iteration as one 16-byte access
+  // `x0 = a[4q]; ...; b[4q] = r0; x1 = a[4q + 1]; ...; b[4q + 1] = r1; ...` (what a loop over the four
+  // elements of a group becomes once it is expanded): the four loads are issued as one vector load where the
+  // first of them stands, the four stores as one vector store where the last of them stands.  The device
+  // compiler does not do this by itself when `a` and `b` are pointers that may name the same array; it is safe
+  // here because an access that changes places only passes accesses to other elements: a store to y[f + c1] and a
+  // load of x[f + c2] with c1 != c2 never touch the same element, whether or not x and y are the same array, and
+  // accesses to LDS and to global memory never do.  On LDS this is the difference between four partial-bank
+  // accesses and one full-rate one per lane.
+  struct Pack { std::string var, decl_ty, addr; bool is_store = false; size_t first = 0, last = 0; const Stmts* owner = nullptr; };
+  std::map<const Expr*, std::string> pack_loads;                   // load expression -> "pk.x"
+  std::map<const Stmt*, std::pair<int, int>> pack_stores;          // store statement -> (pack index, component)
+  std::vector<Pack> packs;
+  int pack_counter = 0;
+
+  static bool multiple_of_four(const E& e) {
+    if (e->k == Expr::Int) return e->iv % 4 == 0;
+    if (e->k == Expr::Convert) return multiple_of_four(e->args[0]);
+    if (e->k != Expr::BinOpE) return false;
+    if (e->bop == BinOp::Mul) return (e->args[0]->k == Expr::Int && e->args[0]->iv % 4 == 0) || (e->args[1]->k == Expr::Int && e->args[1]->iv % 4 == 0);
+    if (e->bop == BinOp::Add || e->bop == BinOp::Sub) return multiple_of_four(e->args[0]) && multiple_of_four(e->args[1]);
+    return false;
+  }
+  // idx == f + c with f a multiple of four and 0 <= c < 4; the constant may sit anywhere in a sum
+  static void sum_terms(const E& e, std::vector<E>& terms, int64_t& c) {
+    if (e->k == Expr::BinOpE && e->bop == BinOp::Add) { sum_terms(e->args[0], terms, c); sum_terms(e->args[1], terms, c); return; }
+    if (e->k == Expr::Int) { c += e->iv; return; }
+    terms.push_back(e);
+  }
+  static bool split_offset(const E& idx, E* f, int64_t* c) {
+    std::vector<E> terms;
+    int64_t k = 0;
+    sum_terms(idx, terms, k);
+    if (terms.empty()) return false;
+    for (auto& t : terms) if (!multiple_of_four(t)) return false;
+    int64_t base = k - (((k % 4) + 4) % 4);
+    E sum = terms[0];
+    for (size_t i = 1; i < terms.size(); ++i) sum = mk_binop(BinOp::Add, sum, terms[i], idx->ty);
+    if (base != 0) sum = mk_binop(BinOp::Add, sum, mk_int(base, idx->ty.sz), idx->ty);
+    *f = sum;
+    *c = k - base;
+    return true;
+  }
+  bool packable(const E& x) const {
+    if (x->k != Expr::Index || x->args[0]->k != Expr::Var || elem_bytes(x->ty.sz) != 4 || !x->ty.is_scalar()) return false;
+    const E& base = x->args[0];
+    if (exchanged(x) || stream_out.count(base->name)) return false;
+    if (base->ty.mem == Mem::LDS) return true;
+    // global: a parameter of a kernel whose pointer arguments are 16-byte aligned
+    if (!kernel->aligned_params) return false;
+    for (auto& p : kernel->params)
+      if (p.id == base->name) return p.ty.k == Type::Pointer;
+    return false;
+  }
+
+  struct Access { size_t pos; const Expr* e; const Stmt* st; bool store; Name base; Mem mem; E f; int64_t c; bool tracked; };
+
+  void plan_packs(const Stmts& ss, size_t lo, size_t hi) {
+    // every element access of the run in program order (an assignment evaluates its right-hand side first)
+    std::vector<Access> acc;
+    for (size_t i = lo; i < hi; ++i) {
+      const S& st = ss[i];
+      auto scan = [&](const E& root) {
+        visit_exprs(root, [&](const E& x) {
+          if (x->k != Expr::Index) return;
+          Access a{i, x.get(), st.get(), false, x->args[0]->k == Expr::Var ? x->args[0]->name : Name(), x->args[0]->ty.mem, E(), 0, false};
+          a.tracked = x->args[0]->k == Expr::Var && split_offset(x->args[1], &a.f, &a.c);
+          acc.push_back(a);
+        });
+      };
+      if (st->expr) scan(st->expr);
+      if (st->k == Stmt::Assign && st->dst->k == Expr::Index) {
+        scan(st->dst->args[1]);
+        Access a{i, st->dst.get(), st.get(), true, st->dst->args[0]->k == Expr::Var ? st->dst->args[0]->name : Name(), st->dst->args[0]->ty.mem, E(), 0, false};
+        a.tracked = st->dst->args[0]->k == Expr::Var && split_offset(st->dst->args[1], &a.f, &a.c);
+        acc.push_back(a);
+      } else if (st->dst) {
+        scan(st->dst);
+      }
+    }
+    auto independent = [&](const Access& a, const Access& b) {
+      if (a.mem != b.mem) return true;                                   // LDS and global memory are disjoint
+      if (a.tracked && b.tracked && expr_eq(a.f, b.f) && a.c != b.c) return true;   // other elements of the same group
+      return false;
+    };
+    auto lookup = [&](const Access& a) -> E {
+      for (size_t i = lo; i < hi; ++i) {
+        E found;
+        auto scan = [&](const E& root) { visit_exprs(root, [&](const E& x) { if (x.get() == a.e) found = x; }); };
+        if (ss[i]->expr) scan(ss[i]->expr);
+        if (ss[i]->dst) scan(ss[i]->dst);
+        if (found) return found;
+      }
+      return E();
+    };
+    std::set<size_t> used;
+    for (size_t i = 0; i < acc.size(); ++i) {
+      const Access& a0 = acc[i];
+      if (used.count(i) || !a0.tracked || a0.c != 0) continue;
+      E e0 = lookup(a0);
+      if (!e0 || !packable(e0)) continue;
+      // the other three elements, same direction, same array, same f
+      size_t member[4] = {i, 0, 0, 0};
+      bool ok = true;
+      for (int64_t c = 1; c < 4 && ok; ++c) {
+        bool found = false;
+        for (size_t j = 0; j < acc.size(); ++j)
+          if (!used.count(j) && acc[j].tracked && acc[j].store == a0.store && acc[j].base == a0.base && acc[j].c == c && expr_eq(acc[j].f, a0.f)) {
+            member[c] = j;
+            found = true;
+            break;
+          }
+        ok = found;
+      }
+      if (!ok) continue;
+      // each element of the array may appear once in the group's direction (a second load of a[4q] keeps its place)
+      size_t first = i, last = i;
+      for (int c = 0; c < 4; ++c) { first = std::min(first, member[c]); last = std::max(last, member[c]); }
+      // loads move up to the first member, stores down to the last: everything passed on the way must be independent
+      for (int c = 0; c < 4 && ok; ++c) {
+        size_t from = a0.store ? member[c] + 1 : first, to = a0.store ? last + 1 : member[c];
+        for (size_t j = from; j < to && ok; ++j) {
+          bool is_member = false;
+          for (int d = 0; d < 4; ++d) is_member = is_member || member[d] == j;
+          if (is_member) continue;
+          // a load passes stores, a store passes loads and stores
+          if (!a0.store && !acc[j].store) continue;
+          if (!independent(acc[member[c]], acc[j])) ok = false;
+        }
+      }
+      // the index of the group must not use anything defined inside the span it moves across
+      if (ok) {
+        std::set<Name> defined;
+        for (size_t s2 = acc[first].pos; s2 <= acc[last].pos && s2 < hi; ++s2)
+          if (ss[s2]->k == Stmt::Def) defined.insert(ss[s2]->id);
+        visit_exprs(a0.f, [&](const E& x) { if (x->k == Expr::Var && defined.count(x->name)) ok = false; });
+      }
+      if (!ok) continue;
+      Pack pk;
+      pk.var = "pk_" + std::to_string(pack_counter++);
+      pk.is_store = a0.store;
+      pk.first = acc[first].pos;
+      pk.last = acc[last].pos;
+      pk.owner = &ss;
+      pk.decl_ty = std::string("parpy_vec4<") + elem_ctype(e0->ty.sz) + ">";
+      as_lvalue = true;
+      std::string elem = pexpr(e0);
+      as_lvalue = false;
+      bool lds_ptr = e0->args[0]->ty.mem == Mem::LDS;
+      pk.addr = std::string("(") + (lds_ptr ? "__attribute__((address_space(3))) " : "") + (a0.store ? "" : "const ") + pk.decl_ty + "*)&" + elem;
+      int pi = (int)packs.size();
+      packs.push_back(pk);
+      static const char* comp = "xyzw";
+      for (int c = 0; c < 4; ++c) {
+        used.insert(member[c]);
+        if (a0.store) pack_stores[acc[member[c]].st] = {pi, c};
+        else pack_loads[acc[member[c]].e] = pk.var + "." + comp[c];
+      }
+    }
+  }
+
   void pstmts(const Stmts& ss, int n) {
-    for (auto& s : ss) pstmt(s, n);
+    size_t first_pack = packs.size();
+    if (opts.opt_pack_accesses && kernel) {
+      // straight-line runs of definitions and assignments
+      for (size_t i = 0; i < ss.size();) {
+        if (!(ss[i]->k == Stmt::Def || ss[i]->k == Stmt::Assign)) { ++i; continue; }
+        size_t j = i;
+        while (j < ss.size() && (ss[j]->k == Stmt::Def || ss[j]->k == Stmt::Assign)) ++j;
+        if (j - i >= 4) plan_packs(ss, i, j);
+        i = j;
+      }
+    }
+    for (size_t i = 0; i < ss.size(); ++i) {
+      for (size_t p = first_pack; p < packs.size(); ++p)
+        if (packs[p].owner == &ss && packs[p].first == i) {
+          if (packs[p].is_store) os << ind(n) << packs[p].decl_ty << " " << packs[p].var << ";\n";
+          else os << ind(n) << "const " << packs[p].decl_ty << " " << packs[p].var << " = *" << packs[p].addr << ";\n";
+        }
+      pstmt(ss[i], n);
+      for (size_t p = first_pack; p < packs.size(); ++p)
+        if (packs[p].owner == &ss && packs[p].is_store && packs[p].last == i) os << ind(n) << "*" << packs[p].addr << " = " << packs[p].var << ";\n";
+    }
   }
 
   std::string kernel_text(const Kernel& k) {
@@ -810,6 +1003,9 @@ struct DevicePrinter {
     narrow_vars.clear();
     reassigned.clear();
     lds_decls.clear();
+    pack_loads.clear();
+    pack_stores.clear();
+    packs.clear();
     os.str("");
     find_reassigned(k.body, reassigned);
     stream_out.clear();

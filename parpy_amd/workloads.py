@@ -8,7 +8,7 @@ HIP backend -- nothing here calls a hand-written kernel.
 import numpy as np
 
 import parpy_amd as parpy
-from parpy_amd.operators import exp, float32, inf, int32, log, max, sum
+from parpy_amd.operators import exp, float32, float64, inf, int32, log, max, sum
 
 
 # ---------------------------------------------------------------- reductions / softmax
@@ -339,6 +339,71 @@ def forward_syn4(hmm, seqs, result, alpha1, alpha2):
         forward_syn_lse(hmm, seqs, result, alpha1, alpha2, inst)
 
 
+# ---------------------------------------------------------------- HMM forward, synthetic model, scaled linear space
+@parpy.jit
+def forward_scaled_step(hmm, seqs, beta1, beta2, inst, t):
+    beta_src = beta2
+    beta_dst = beta1
+    if t & 1:
+        beta_src = beta1
+        beta_dst = beta2
+    o = seqs["data"][inst, t]
+    parpy.label('state')
+    for q in range(hmm["num_states"] // 4):
+        if t < seqs["lens"][inst]:
+            nq = hmm["num_states"] // 4
+            a1 = beta_src[inst, q]
+            a2 = beta_src[inst, nq + q]
+            a3 = beta_src[inst, 2 * nq + q]
+            a4 = beta_src[inst, 3 * nq + q]
+            for u in range(4):
+                s = (a1 * hmm["ptrans1"][q, u] + a2 * hmm["ptrans1"][nq + q, u] +
+                     a3 * hmm["ptrans1"][2 * nq + q, u] + a4 * hmm["ptrans1"][3 * nq + q, u] +
+                     beta_src[inst, 4 * q + u] * hmm["pstay"][4 * q + u])
+                beta_dst[inst, 4 * q + u] = s * hmm["pemit"][o, 4 * q + u]
+
+
+@parpy.jit
+def forward_scaled_renorm(hmm, seqs, beta1, beta2, inst, t):
+    beta = beta1
+    if t & 1:
+        beta = beta2
+    parpy.label('state')
+    top = max(beta[inst, :])
+    parpy.label('state')
+    beta[inst, :] = beta[inst, :] * (float32(1.0) / top)
+    return log(float64(top))
+
+
+@parpy.jit
+def forward_scaled(hmm, seqs, result, beta1, beta2):
+    """The forward pass of the synthetic model in linear space with rescaling (the classical alternative to
+    log space): beta[s] holds the probability alpha[s] times a running scale whose logarithm is kept in
+    float64.  Tables are probabilities: `ptrans1`, `pstay`, `pinit`, and `pemit` = emission probabilities
+    times the constant exp(`log_emit_scale`) that makes the largest of them one.  A step is five multiply-adds
+    and one multiplication per state, no exponential and no logarithm; every eighth step the state vector is
+    divided by its largest element.  The result is float64:
+    log-likelihood = log(sum of the final vector) + sum of log(divisors) - len * log_emit_scale."""
+    parpy.label('inst')
+    for inst in range(seqs["num_instances"]):
+        o0 = seqs["data"][inst, 0]
+        parpy.label('state')
+        for state in range(hmm["num_states"]):
+            beta1[inst, state] = hmm["pinit"][state] * hmm["pemit"][o0, state]
+        scale = float64(0.0)
+        for t in range(1, seqs["maxlen"]):
+            forward_scaled_step(hmm, seqs, beta1, beta2, inst, t)
+            if t < seqs["lens"][inst]:
+                if t % 8 == 0:
+                    scale = scale + forward_scaled_renorm(hmm, seqs, beta1, beta2, inst, t)
+        beta = beta1
+        if seqs["lens"][inst] & 1 == 0:
+            beta = beta2
+        parpy.label('state')
+        total = sum(beta[inst, :])
+        result[inst] = scale + log(float64(total)) - float64(seqs["lens"][inst]) * hmm["log_emit_scale"]
+
+
 # ---------------------------------------------------------------- seeded inputs
 SEED = 1234
 
@@ -454,6 +519,18 @@ def with_linear_tables(hmm):
     out = dict(hmm)
     out["ptrans1"] = np.exp(hmm["trans1"].astype(np.float64)).astype(np.float32)
     out["pstay"] = np.exp(hmm["stay"].astype(np.float64)).astype(np.float32)
+    return out
+
+
+def with_scaled_tables(hmm):
+    """The model with probability tables for `forward_scaled`: `ptrans1`, `pstay`, `pinit`, and the emission
+    probabilities times one constant that makes the largest of them one (`pemit`; `log_emit_scale` is the
+    logarithm of that constant, a Python float and so a compile-time constant of the kernel)."""
+    out = with_linear_tables(hmm)
+    out["pinit"] = np.exp(hmm["initial_prob"].astype(np.float64)).astype(np.float32)
+    e = hmm["output_prob"].astype(np.float64)
+    out["log_emit_scale"] = float(-e.max())
+    out["pemit"] = np.exp(e + out["log_emit_scale"]).astype(np.float32)
     return out
 
 
