@@ -11,12 +11,14 @@ under `secondary` of the same JSON line.  Every record carries the roofline of
 its dominant kernel (algorithmic bytes or flops / measured kernel time against
 the published peak) and a CPU baseline timed on the host cores (bounded sample).
 
-The HMM forward pass is timed in two forms of the same recurrence, both written
-as ParPy user code in parpy_amd/workloads.py: `grouped` (forward_syn4: the four
-states that share their predecessors are updated together, `value` of the
-headline) and `reference` (forward_syn: one state at a time, the structure of
-the reference's kernel); the figure of the other form is in the record too.
-Results are checked against the oracle outside the timed region.
+The HMM forward pass is timed in three statements of the same recurrence, all
+written as ParPy user code in parpy_amd/workloads.py: `scaled` (forward_scaled:
+linear space with rescaling, float64 result, the one that meets the 1e-4
+tolerance against the fp64 oracle and the `value` of the headline), `grouped`
+(forward_syn4: log space, the four states that share their predecessors updated
+together) and `reference` (forward_syn: log space, one state at a time, the
+structure of the reference's kernel).  The figures of the other forms are in
+the record too.  Results are checked against the oracle outside the timed region.
 """
 import argparse
 import json
@@ -42,8 +44,10 @@ OPT_FLAGS = ("opt_vectorize", "opt_lds_rows", "opt_reg_cache", "opt_hoist_invari
 VALU_NS = {"full": 1.17, "trans": 3.76}
 HMM_VALU_MIX = {
     "reference": {"full": 24.0, "trans": 6.0},
-    "grouped": {"full": 16.75, "trans": 3.0},
+    "grouped": {"full": 14.2, "trans": 3.0},
+    "scaled": {"full": 7.5, "trans": 0.0},
 }
+HMM_FORMS = {"scaled": "forward_scaled", "grouped": "forward_syn4", "reference": "forward_syn"}
 
 
 def _events_ms(fn, timed, steps, warmup, torch):
@@ -70,9 +74,9 @@ def _hbm_roofline(alg_bytes, kernel_ms, workload, default_cfg):
 def _time_hmm_form(form, hd, sd, n, S, nthreads, args, torch, parpy, W):
     a1 = torch.zeros((n, S), dtype=torch.float32, device="cuda")
     a2 = torch.zeros_like(a1)
-    res = torch.zeros(n, dtype=torch.float32, device="cuda")
-    f = W.forward_syn4 if form == "grouped" else W.forward_syn
-    threads = min(nthreads, S // 4) if form == "grouped" else min(nthreads, S)
+    res = torch.zeros(n, dtype=torch.float64 if form == "scaled" else torch.float32, device="cuda")
+    f = getattr(W, HMM_FORMS[form])
+    threads = min(nthreads, S) if form == "reference" else min(nthreads, S // 4)
     opts = parpy.par({"inst": parpy.threads(n), "state": parpy.threads(threads)})
     _apply_opt_flags(opts, args)
     opts.use_cuda_graphs = bool(args.use_graphs)
@@ -89,14 +93,14 @@ def bench_hmm(k, args, torch, parpy, W, default_cfg=True):
     import oracle
     hmm, seqs = W.synthetic_hmm(k)
     S, n = hmm["num_states"], seqs["num_instances"]
-    hd, sd = W.to_device(W.with_linear_tables(hmm)), W.to_device(seqs)
+    hd, sd = W.to_device(W.with_scaled_tables(hmm)), W.to_device(seqs)
     steps_total = int((seqs["lens"] - 1).sum())
     longest = int(seqs["lens"].max()) - 1
     # per (sequence, step): read alpha (4S) + write alpha (4S) + emission row (4S) + the observation byte
     alg_bytes = (12 * S + 1) * steps_total
-    other = "reference" if args.form == "grouped" else "grouped"
+    others = [f for f in ("scaled", "grouped", "reference") if f != args.form]
     forms = {}
-    for form in (args.form, other):
+    for form in [args.form] + others:
         wall, kernel_ms, ll, threads = _time_hmm_form(form, hd, sd, n, S, args.state_threads, args, torch, parpy, W)
         mix = HMM_VALU_MIX[form]
         rows_per_simd = S / 256.0
@@ -111,7 +115,9 @@ def bench_hmm(k, args, torch, parpy, W, default_cfg=True):
     checked = {}
     for form, r in forms.items():
         err = float(np.abs(r["ll"][sub].astype(np.float64) - want).max())
-        assert np.all(np.isfinite(r["ll"])) and err < 0.2, f"{form} form of the {k}-mer forward pass is off by {err}"
+        # the scaled form is held to the 1e-4 of the workload's definition, the fp32 log-space forms to their measured drift
+        limit = 1e-4 if form == "scaled" else 0.2
+        assert np.all(np.isfinite(r["ll"])) and err < limit, f"{form} form of the {k}-mer forward pass is off by {err}"
         checked[form] = err
     cpu = None
     if not args.no_cpu:
@@ -123,23 +129,30 @@ def bench_hmm(k, args, torch, parpy, W, default_cfg=True):
         cpu = {"value": dt * 1e3 * steps_total / done, "unit": "ms/batch", "cores": os.cpu_count(), "kind": "port",
                "sample": f"first {sample_steps} samples of each of the {n} reads with the C oracle "
                          f"(OpenMP over reads), {dt:.1f} s measured, scaled by total steps {steps_total}/{done}"}
-    main, alt = forms[args.form], forms[other]
-    name = {"grouped": "forward_syn4", "reference": "forward_syn"}
-    roof = _hbm_roofline(alg_bytes, main["kernel_ms"], f"hmm{k}" + ("_grouped" if args.form == "grouped" else ""), default_cfg)
+    main = forms[args.form]
+    name = HMM_FORMS
+    suffix = {"scaled": "_scaled", "grouped": "_grouped", "reference": ""}
+    roof = _hbm_roofline(alg_bytes, main["kernel_ms"], f"hmm{k}{suffix[args.form]}", default_cfg)
     roof["valu_bound"] = main["valu_bound"]
-    alt_roof = _hbm_roofline(alg_bytes, alt["kernel_ms"], f"hmm{k}" + ("_grouped" if other == "grouped" else ""), default_cfg)
-    alt_roof["valu_bound"] = alt["valu_bound"]
+    other_forms = []
+    for other in others:
+        alt = forms[other]
+        alt_roof = _hbm_roofline(alg_bytes, alt["kernel_ms"], f"hmm{k}{suffix[other]}", default_cfg)
+        alt_roof["valu_bound"] = alt["valu_bound"]
+        other_forms.append({"form": f"{other} ({name[other]})", "ms_per_step": alt["wall"], "state_threads": alt["threads"],
+                            "dtype": "f32 state vectors, " + ("f64 result" if other == "scaled" else "f32 result"),
+                            "roofline": alt_roof, "checked_max_abs_error": checked[other]})
     return {
         "metric": f"HMM-forward {k}-mer ms/batch + achieved HBM GB/s (% of peak), 1xMI355X",
         "value": main["wall"], "unit": "ms/batch", "ms_per_step": main["wall"], "higher_is_better": False,
         "dtype": "f32",
-        "config": {"workload": f"hmm_forward_{k}mer_synthetic", "form": f"{args.form} ({name[args.form]})", "states": S, "reads": n,
+        "config": {"workload": f"hmm_forward_{k}mer_synthetic", "form": f"{args.form} ({name[args.form]})",
+                   "result_dtype": "f64" if args.form == "scaled" else "f32", "states": S, "reads": n,
                    "min_len": 5000, "max_len": 15000, "total_steps": steps_total, "state_threads": main["threads"],
                    "graph_replay": bool(args.use_graphs), "mean_loglik": float(main["ll"].mean()),
                    "checked": f"6 shortest reads at full length against the fp64 oracle, max abs error {checked[args.form]:.3g}"},
         "roofline": roof,
-        "other_form": {"form": f"{other} ({name[other]})", "ms_per_step": alt["wall"], "state_threads": alt["threads"],
-                       "roofline": alt_roof, "checked_max_abs_error": checked[other]},
+        "other_forms": other_forms,
         "cpu_baseline": cpu,
     }
 
@@ -355,8 +368,8 @@ def main():
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="all", choices=["all", "hmm7", "hmm5", "hmm5ref", "rowsum", "softmax", "sddmm", "copy"])
-    ap.add_argument("--form", default="grouped", choices=["grouped", "reference"],
-                    help="which statement of the HMM step is the record's value (the other is timed beside it)")
+    ap.add_argument("--form", default="scaled", choices=["scaled", "grouped", "reference"],
+                    help="which statement of the HMM step is the record's value (the others are timed beside it)")
     ap.add_argument("--state-threads", type=int, default=1024)
     ap.add_argument("--use-graphs", type=int, default=0, help="replay the launches of a run from a HIP graph (host-hoisted time loops)")
     ap.add_argument("--persistent", type=int, default=0, help="run host-hoisted time loops inside one kernel when the grid fits the device")

@@ -299,6 +299,17 @@ def _run_grouped(hmm, seqs, threads, **kw):
     return res.cpu().numpy(), a1.cpu().numpy(), a2.cpu().numpy()
 
 
+def _run_scaled(hmm, seqs, threads, **kw):
+    """`forward_scaled`: linear space with rescaling, float64 result."""
+    hd, sd = W.to_device(W.with_scaled_tables(hmm)), W.to_device(seqs)
+    n, S = seqs["num_instances"], hmm["num_states"]
+    b1 = torch.zeros((n, S), dtype=torch.float32, device="cuda")
+    b2 = torch.zeros_like(b1)
+    res = torch.zeros(n, dtype=torch.float64, device="cuda")
+    W.forward_scaled(hd, sd, res, b1, b2, opts=opts_for({'inst': parpy.threads(n), 'state': parpy.threads(threads)}, **kw))
+    return res.cpu().numpy()
+
+
 _FULL = {}
 
 
@@ -313,6 +324,8 @@ def _full_size(k, what):
             _FULL[(what, k)] = _run_synthetic(hmm, seqs, min(1024, hmm["num_states"]))[0]
         elif what == "forward_syn4":
             _FULL[(what, k)] = _run_grouped(hmm, seqs, min(1024, hmm["num_states"] // 4))[0]
+        elif what == "forward_scaled":
+            _FULL[(what, k)] = _run_scaled(hmm, seqs, min(1024, hmm["num_states"] // 4))
         else:
             _FULL[(what, k)] = oracle.hmm_syn_forward(hmm, seqs, what)
     return _FULL[(what, k)]
@@ -323,17 +336,22 @@ def _full_size(k, what):
 # magnitude.  The fp32 oracle runs the reference's operation order, so `forward_syn` stays within an ulp or two
 # of it while both drift from fp64 by the rounding of 15000 dependent log-space steps; `forward_syn4` rounds
 # differently (fewer, larger terms per step) and lands closer to fp64 than the fp32 oracle does on the 5-mer.
+# `forward_scaled` works in linear space with the scale kept in float64 and returns float64: it is the form that
+# meets the 1e-4 bar against the fp64 oracle (measured 6.1e-6 and 3.6e-6); against the fp32 oracle it shows that
+# oracle's own drift.
 FULL_SIZE_BOUNDS = {
     # (k, form): (measured vs fp32 oracle, bound, measured vs fp64 oracle, bound)
     (5, "forward_syn"): (0.0078, 0.02, 0.339, 0.5),
     (5, "forward_syn4"): (0.387, 0.6, 0.0593, 0.1),
     (7, "forward_syn"): (0.0039, 0.02, 0.0299, 0.06),
     (7, "forward_syn4"): (0.0391, 0.08, 0.0423, 0.08),
+    (5, "forward_scaled"): (0.339, 0.5, 6.1e-6, 1e-4),
+    (7, "forward_scaled"): (0.0299, 0.06, 3.6e-6, 1e-4),
 }
 
 
 @pytest.mark.parametrize("prec", [np.float32, np.float64], ids=["fp32-oracle", "fp64-oracle"])
-@pytest.mark.parametrize("form", ["forward_syn", "forward_syn4"])
+@pytest.mark.parametrize("form", ["forward_syn", "forward_syn4", "forward_scaled"])
 @pytest.mark.parametrize("k", [5, 7])
 def test_forward_full_size_every_read_against_the_oracle(k, form, prec):
     """BASELINE configurations 4 and 5 at full size: every one of the 100 reads against the fp32 and the fp64
@@ -350,6 +368,49 @@ def test_forward_full_size_every_read_against_the_oracle(k, form, prec):
     assert np.allclose(got, want, atol=1e-5, rtol=1e-5)
 
 
+@pytest.mark.parametrize("k,threads", [(3, 64), (4, 64), (5, 64), (5, 256), (6, 1024), (7, 1024)])
+def test_forward_scaled_vs_oracle(k, threads):
+    """Linear space with rescaling against the fp64 oracle, to north_star's 1e-4 absolute: reads of one sample (no
+    step), of eight (no rescaling yet), of nine (rescaled once) and up to 300."""
+    hmm, seqs = W.synthetic_hmm(k, n_inst=16, min_len=1, max_len=300)
+    seqs["lens"][:4] = [1, 8, 9, 17]
+    got = _run_scaled(hmm, seqs, threads)
+    want = oracle.hmm_syn_forward(hmm, seqs, np.float64)
+    assert np.abs(got - want).max() < 1e-4, np.abs(got - want).max()
+
+
+@pytest.mark.parametrize("flags", [{"opt_pack_accesses": False}, {"opt_prefetch_steps": False}, {"opt_expand_short_loops": False},
+                                   {"opt_guard_bounds": False}, {"opt_hoist_invariant": False}, {"opt_lds_rows": False}],
+                         ids=lambda f: ",".join(f"{k}={int(v)}" for k, v in f.items()))
+def test_forward_scaled_each_pass_preserves_results(flags):
+    hmm, seqs = W.synthetic_hmm(5, n_inst=8, min_len=50, max_len=200)
+    base = _run_scaled(hmm, seqs, 256)
+    got = _run_scaled(hmm, seqs, 256, **flags)
+    want = oracle.hmm_syn_forward(hmm, seqs, np.float64)
+    assert np.abs(got - want).max() < 1e-4
+    assert np.abs(got - base).max() < 1e-5
+
+
+def test_forward_scaled_unreachable_and_improbable_states():
+    """Probability zero is exact in linear space (log 0 = -inf only if every state is unreachable); a start that is
+    e^-400 less likely than the others is below what fp32 holds next to them and counts as zero, which moves the
+    result by less than the tolerance."""
+    hmm, seqs = W.synthetic_hmm(4, n_inst=6, min_len=3, max_len=60, seed=7)
+    rng = np.random.default_rng(3)
+    S = hmm["num_states"]
+    init = hmm["initial_prob"].copy()
+    init[rng.random(S) < 0.4] = -400.0
+    init[rng.random(S) < 0.2] = -np.inf
+    init[5] = 0.0
+    hmm["initial_prob"] = init.astype(np.float32)
+    got = _run_scaled(hmm, seqs, 64)
+    want = oracle.hmm_syn_forward(hmm, seqs, np.float64)
+    assert np.all(np.isfinite(want)) and np.abs(got - want).max() < 1e-4
+    hmm["initial_prob"][:] = -np.inf
+    got = _run_scaled(hmm, seqs, 64)
+    assert np.all(np.isneginf(got) | np.isnan(got))
+
+
 def test_forward_7mer_constant_emissions_closed_form():
     """Constant emissions: the log-likelihood is len * c whatever the transitions are (full headline shape)."""
     c = np.float32(np.log(1.0 / 101.0))
@@ -360,6 +421,10 @@ def test_forward_7mer_constant_emissions_closed_form():
     assert np.allclose(got_c, seqs_c["lens"] * float(c), rtol=5e-4, atol=0)
     got_g, _, _ = _run_grouped(hmm_c, seqs_c, 1024)
     assert np.allclose(got_g, seqs_c["lens"] * float(c), rtol=5e-4, atol=0)
+    # in linear space the only rounding is that of the sums of transition probabilities (each state's incoming
+    # mass is not one, only the outgoing mass is): far below the tolerance of the log-space forms
+    got_s = _run_scaled(hmm_c, seqs_c, 1024)
+    assert np.allclose(got_s, seqs_c["lens"] * float(c), rtol=1e-7, atol=1e-3), np.abs(got_s - seqs_c["lens"] * float(c)).max()
 
 
 @pytest.mark.parametrize("k,threads", [(3, 64), (4, 64), (5, 64), (5, 256), (6, 1024), (5, 1024)])
