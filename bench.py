@@ -98,7 +98,7 @@ def bench_hmm(k, args, torch, parpy, W, default_cfg=True):
     longest = int(seqs["lens"].max()) - 1
     # per (sequence, step): read alpha (4S) + write alpha (4S) + emission row (4S) + the observation byte
     alg_bytes = (12 * S + 1) * steps_total
-    others = [f for f in ("scaled", "grouped", "reference") if f != args.form]
+    others = [] if args.single_form else [f for f in ("scaled", "grouped", "reference") if f != args.form]
     forms = {}
     for form in [args.form] + others:
         wall, kernel_ms, ll, threads = _time_hmm_form(form, hd, sd, n, S, args.state_threads, args, torch, parpy, W)
@@ -370,6 +370,7 @@ def main():
     ap.add_argument("--workload", default="all", choices=["all", "hmm7", "hmm5", "hmm5ref", "rowsum", "softmax", "sddmm", "copy"])
     ap.add_argument("--form", default="scaled", choices=["scaled", "grouped", "reference"],
                     help="which statement of the HMM step is the record's value (the others are timed beside it)")
+    ap.add_argument("--single-form", action="store_true", help="time only the chosen form of the HMM step (profiling runs)")
     ap.add_argument("--state-threads", type=int, default=1024)
     ap.add_argument("--use-graphs", type=int, default=0, help="replay the launches of a run from a HIP graph (host-hoisted time loops)")
     ap.add_argument("--persistent", type=int, default=0, help="run host-hoisted time loops inside one kernel when the grid fits the device")
