@@ -821,7 +821,7 @@ struct DevicePrinter {
   // load of x[f + c2] with c1 != c2 never touch the same element, whether or not x and y are the same array, and
   // accesses to LDS and to global memory never do.  On LDS this is the difference between four partial-bank
   // accesses and one full-rate one per lane.
-  struct Pack { std::string var, decl_ty, addr; bool is_store = false; size_t first = 0, last = 0; const Stmts* owner = nullptr; };
+  struct Pack { std::string var, decl_ty, addr; bool is_store = false, streamed = false; size_t first = 0, last = 0; const Stmts* owner = nullptr; };
   std::map<const Expr*, std::string> pack_loads;                   // load expression -> "pk.x"
   std::map<const Stmt*, std::pair<int, int>> pack_stores;          // store statement -> (pack index, component)
   std::vector<Pack> packs;
@@ -858,7 +858,7 @@ struct DevicePrinter {
   bool packable(const E& x) const {
     if (x->k != Expr::Index || x->args[0]->k != Expr::Var || elem_bytes(x->ty.sz) != 4 || !x->ty.is_scalar()) return false;
     const E& base = x->args[0];
-    if (exchanged(x) || stream_out.count(base->name)) return false;
+    if (exchanged(x)) return false;
     if (base->ty.mem == Mem::LDS) return true;
     // global: a parameter of a kernel whose pointer arguments are 16-byte aligned
     if (!kernel->aligned_params) return false;
@@ -956,6 +956,7 @@ struct DevicePrinter {
       pk.first = acc[first].pos;
       pk.last = acc[last].pos;
       pk.owner = &ss;
+      pk.streamed = a0.store && stream_out.count(a0.base) > 0;   // write-once data keeps bypassing the caches
       pk.decl_ty = std::string("parpy_vec4<") + elem_ctype(e0->ty.sz) + ">";
       as_lvalue = true;
       std::string elem = pexpr(e0);
@@ -993,7 +994,10 @@ struct DevicePrinter {
         }
       pstmt(ss[i], n);
       for (size_t p = first_pack; p < packs.size(); ++p)
-        if (packs[p].owner == &ss && packs[p].is_store && packs[p].last == i) os << ind(n) << "*" << packs[p].addr << " = " << packs[p].var << ";\n";
+        if (packs[p].owner == &ss && packs[p].is_store && packs[p].last == i) {
+          if (packs[p].streamed) os << ind(n) << "__builtin_nontemporal_store(" << packs[p].var << ", " << packs[p].addr << ");\n";
+          else os << ind(n) << "*" << packs[p].addr << " = " << packs[p].var << ";\n";
+        }
     }
   }
 

@@ -282,6 +282,54 @@ def test_loop_bound_from_guard_needs_every_effect_under_the_guard():
     assert "t_end_" not in s
 
 
+def test_scaled_hmm_step_packs_its_lds_accesses_and_fetches_the_emission_row_a_step_ahead():
+    hmm, seqs, args = _hmm_args(5)
+    args = [W.with_scaled_tables(args[0]), args[1], np.zeros(4, dtype=np.float64)] + args[3:]
+    o = opts_for({'inst': parpy.threads(4), 'state': parpy.threads(64)})
+    s = compiles(parpy.print_compiled(W.forward_scaled, args, o))
+    step = s[s.index("for (int t_"):]
+    step = step[:step.index("__syncthreads")]
+    # the observation of the next step is loaded while this one runs, and with it the thread's part of the emission row
+    assert re.search(r"int8_t o_\d+ = o_next_\d+;\n\s+o_next_\d+ = seqs_data_\d+\[", step)
+    assert len(re.findall(r"float row_hmm_pemit_\d+\[4\];", s)) == 4
+    assert len(re.findall(r"row_hmm_pemit_\d+\[q_\d+_k\] = pk_\d+\.[xyzw];", step)) == 4      # refilled from one 16-byte load
+    # own states: one 16-byte LDS load; results: one 16-byte LDS store
+    assert re.search(r"const parpy_vec4<float> pk_\d+ = \*\(__attribute__\(\(address_space\(3\)\)\) const parpy_vec4<float>\*\)&beta_src_\d+\[\(4 \* q_\d+\)\];", step)
+    assert re.search(r"\*\(__attribute__\(\(address_space\(3\)\)\) parpy_vec4<float>\*\)&beta_dst_\d+\[\(4 \* q_\d+\)\] = pk_\d+;", step)
+    assert "__builtin_amdgcn_exp2f" not in step and "__builtin_amdgcn_logf" not in step
+    s0 = compiles(parpy.print_compiled(W.forward_scaled, args, opts_for({'inst': parpy.threads(4), 'state': parpy.threads(64)},
+                                                                          opt_pack_accesses=False, opt_prefetch_steps=False)))
+    assert "pk_" not in s0 and "o_next" not in s0 and "row_hmm_pemit" not in s0
+
+
+def test_adjacent_accesses_are_only_packed_when_nothing_they_pass_can_touch_them():
+    @parpy.jit
+    def shift_groups(a, b, N):
+        parpy.label('i')
+        for q in range(N):
+            b[4 * q] = a[4 * q] + 1.0
+            b[4 * q + 1] = a[4 * q + 1] + 1.0
+            b[4 * q + 2] = a[4 * q + 2] + 1.0
+            b[4 * q + 3] = a[4 * q + 3] + 1.0
+
+    @parpy.jit
+    def carry_groups(a, N):
+        parpy.label('i')
+        for q in range(N):
+            a[4 * q + 1] = a[4 * q] + 1.0          # the next load reads what this stores: the loads keep their places
+            a[4 * q + 2] = a[4 * q + 1] + 1.0
+            a[4 * q + 3] = a[4 * q + 2] + 1.0
+            a[4 * q] = a[4 * q + 3] + 1.0
+    a, b = np.zeros(4096, dtype=np.float32), np.zeros(4096, dtype=np.float32)
+    o = opts_for({'i': parpy.threads(1024)})
+    s = compiles(parpy.print_compiled(shift_groups, [a, b, 1024], o))
+    assert len(re.findall(r"const parpy_vec4<float> pk_\d+ = ", s)) == 1
+    # the result array is written once and never read: its one 16-byte store still bypasses the caches
+    assert len(re.findall(r"__builtin_nontemporal_store\(pk_\d+, \(parpy_vec4<float>\*\)&b_\d+\[", s)) == 1
+    s = compiles(parpy.print_compiled(carry_groups, [a, 1024], o))
+    assert "const parpy_vec4<float>" not in s
+
+
 def test_noalias_scope_wraps_the_step_body_when_aliases_never_coincide():
     hmm, seqs, args = _hmm_args(4)
     o = opts_for({'inst': parpy.threads(4), 'state': parpy.threads(256)}, opt_noalias_scopes=True)

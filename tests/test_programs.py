@@ -240,3 +240,43 @@ def test_stencil_and_products_on_slices():
     out = np.zeros((10, 15), dtype=np.float32)
     parpy.jit(mul_planes)(x, y, out, opts=opts_for({'N': parpy.threads(64), 'M': parpy.threads(64)}))
     assert np.array_equal(out, x[:, 0, :] * y[0, :, :])
+
+
+def shift_groups(a, b, N):
+    parpy.label('i')
+    for q in range(N):
+        b[4 * q] = a[4 * q] + 1.0
+        b[4 * q + 1] = a[4 * q + 1] * 2.0
+        b[4 * q + 2] = a[4 * q + 2] - 3.0
+        b[4 * q + 3] = a[4 * q + 3] * a[4 * q]
+
+
+def carry_groups(a, N):
+    parpy.label('i')
+    for q in range(N):
+        a[4 * q + 1] = a[4 * q] + 1.0
+        a[4 * q + 2] = a[4 * q + 1] * 2.0
+        a[4 * q + 3] = a[4 * q + 2] - 3.0
+        a[4 * q] = a[4 * q + 3] * 0.5
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("pack", [True, False], ids=["packed", "unpacked"])
+def test_groups_of_four_adjacent_elements(pack):
+    """Four neighbouring elements read and written by one lane: as one 16-byte access where nothing
+    in between can touch them, element by element where each load reads what the last store wrote."""
+    rng = np.random.default_rng(21)
+    N = 3000
+    a = rng.standard_normal(4 * N).astype(np.float32)
+    b = np.zeros_like(a)
+    o = opts_for({'i': parpy.threads(N)}, opt_pack_accesses=pack)
+    parpy.jit(shift_groups)(a, b, N, opts=o)
+    g = a.reshape(N, 4)
+    want = np.stack([g[:, 0] + np.float32(1), g[:, 1] * np.float32(2), g[:, 2] - np.float32(3), g[:, 3] * g[:, 0]], axis=1)
+    assert np.array_equal(b.reshape(N, 4), want)
+    c = a.copy()
+    parpy.jit(carry_groups)(c, N, opts=o)
+    w1 = g[:, 0] + np.float32(1)
+    w2 = w1 * np.float32(2)
+    w3 = w2 - np.float32(3)
+    assert np.array_equal(c.reshape(N, 4), np.stack([w3 * np.float32(0.5), w1, w2, w3], axis=1))
