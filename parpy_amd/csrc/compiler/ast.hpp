@@ -411,6 +411,7 @@ struct Kernel {
   bool cached_stores = false;   // what this kernel writes is read by the next one: no non-temporal stores
   bool opaque_body = false;     // the body is a call of a device helper: parameters are described by the creator
   bool no_restrict = false;     // workgroups exchange data through the parameters during the kernel: no no-alias promise
+  std::vector<std::vector<Name>> distinct_pointers;  // local pointer variables that never name the same array while both are in scope
 };
 
 struct Program {

@@ -247,11 +247,61 @@ struct Pass {
     return true;
   }
 
-  Stmts expand_short_loops(const Stmts& ss, bool in_par) {
+  // Local names that are defined once with a literal value (`nq = hmm["num_states"] // 4` after the shapes
+  // are known) stand for that value wherever they are read: index arithmetic written with them folds like
+  // arithmetic written with the numbers, which the passes that compare offsets rely on.
+  Stmts propagate_constants(const Stmts& ss) {
+    std::set<Name> reassigned;
+    visit_stmts(ss, [&](const S& c) {
+      if (c->k == Stmt::Assign && c->dst->k == Expr::Var) reassigned.insert(c->dst->name);
+    });
+    std::map<Name, E> env;
+    std::function<Stmts(const Stmts&)> run = [&](const Stmts& b) {
+      Stmts out;
+      for (auto& c : b) {
+        auto fix = [&](const E& e) {
+          if (env.empty()) return e;
+          return fold_expr(rewrite_expr(e, [&](const E& x) -> E {
+            if (x->k != Expr::Var) return x;
+            auto it = env.find(x->name);
+            return it == env.end() ? x : it->second;
+          }));
+        };
+        auto r = std::const_pointer_cast<Stmt>(std::static_pointer_cast<const Stmt>(map_exprs(c, fix)));
+        if (r->k == Stmt::Def && r->expr && r->ty.is_scalar() && !reassigned.count(r->id) &&
+            (r->expr->k == Expr::Int || r->expr->k == Expr::Float || r->expr->k == Expr::Bool) && r->expr->ty == r->ty) {
+          env[r->id] = r->expr;   // (the definition itself stays: it is what the listing shows for the name)
+        }
+        r->body = run(c->body);
+        r->els = run(c->els);
+        out.push_back(r);
+      }
+      return out;
+    };
+    return run(ss);
+  }
+
+  static size_t count_stmts(const Stmts& ss) {
+    size_t n = 0;
+    visit_stmts(ss, [&](const S&) { ++n; });
+    return n;
+  }
+
+  Stmts expand_short_loops(const Stmts& ss0, bool in_par) {
+    // inner loops first: a short loop around a short loop is straight-line code once the inner one is expanded
+    Stmts ss;
+    for (auto& s : ss0) {
+      if (s->body.empty() && s->els.empty()) { ss.push_back(s); continue; }
+      auto r = clone(s);
+      bool par = in_par || (s->k == Stmt::For && s->map.k != GpuMap::None);
+      r->body = expand_short_loops(s->body, par);
+      r->els = expand_short_loops(s->els, par);
+      ss.push_back(r);
+    }
     Stmts out;
     for (auto& s : ss) {
       int64_t n = s->k == Stmt::For && s->map.k == GpuMap::None ? const_extent(s) : -1;
-      if (in_par && n >= 1 && n <= 8 && straight_line(s->body)) {
+      if (in_par && n >= 1 && n <= 8 && straight_line(s->body) && count_stmts(s->body) * (size_t)n <= 256) {
         std::vector<Name> locals;
         visit_stmts(s->body, [&](const S& c) { if (c->k == Stmt::Def) locals.push_back(c->id); });
         for (int64_t it = 0; it < n; ++it) {
@@ -288,11 +338,7 @@ struct Pass {
         }
         continue;
       }
-      auto r = clone(s);
-      bool par = in_par || (s->k == Stmt::For && s->map.k != GpuMap::None);
-      r->body = expand_short_loops(s->body, par);
-      r->els = expand_short_loops(s->els, par);
-      out.push_back(r);
+      out.push_back(s);
     }
     return out;
   }
@@ -1906,12 +1952,14 @@ struct Pass {
     return false;
   }
 
-  Stmts noalias_scopes(const Stmts& ss) {
+  // With `wrap` the rest of the block goes into a scope whose pointer parameters carry the promise; without it the
+  // kernel only records which local pointers never coincide (the printer's access packing asks).
+  Stmts noalias_scopes(const Stmts& ss, bool wrap) {
     Stmts cur;
     for (auto& s : ss) {
       auto r = clone(s);
-      r->body = noalias_scopes(s->body);
-      r->els = noalias_scopes(s->els);
+      r->body = noalias_scopes(s->body, wrap);
+      r->els = noalias_scopes(s->els, wrap);
       cur.push_back(r);
     }
     // the first run of alias-only statements of this block
@@ -1946,12 +1994,12 @@ struct Pass {
     visit_stmts(rest, [&](const S& st) {
       if (st->k == Stmt::Def && (targets.count(st->id) || std::count(order.begin(), order.end(), st->id))) clean = false;
       if (st->k == Stmt::Assign && st->dst->k == Expr::Var && std::count(order.begin(), order.end(), st->dst->name)) clean = false;
-      if ((st->k == Stmt::Def || (st->k == Stmt::Assign && st->dst->k == Expr::Var)) && is_alias_type(st->k == Stmt::Def ? st->ty : st->dst->ty))
+      if (wrap && (st->k == Stmt::Def || (st->k == Stmt::Assign && st->dst->k == Expr::Var)) && is_alias_type(st->k == Stmt::Def ? st->ty : st->dst->ty))
         clean = false;  // a further alias inside the scope could name the same arrays
       auto scan = [&](const E& e) {
         visit_exprs(e, [&](const E& x) {
           if (x->k != Expr::Var) return;
-          if (targets.count(x->name)) clean = false;
+          if (wrap && targets.count(x->name)) clean = false;
           if (std::count(order.begin(), order.end(), x->name)) types[x->name] = x->ty;
         });
       };
@@ -1963,6 +2011,12 @@ struct Pass {
     for (auto& n : order)
       if (types.count(n) && types[n].k == Type::Pointer) params.push_back(mk_var(n, types[n]));
     if (params.size() < 2) return cur;
+    if (!wrap) {
+      std::vector<Name> group;
+      for (auto& e : params) group.push_back(e->name);
+      k.distinct_pointers.push_back(group);
+      return cur;
+    }
     auto scope = std::make_shared<Stmt>();
     scope->k = Stmt::Scope;
     scope->args = params;
@@ -2667,6 +2721,7 @@ void hip_optimize(Program& p, const Options& opts, NameGen& gen) {
     Pass pass(k, opts, gen);
     if (opts.opt_unswitch) pass.unswitch_aliases();
     if (opts.opt_mfma_sddmm) k.body = pass.mfma_dot(k.body);
+    k.body = pass.propagate_constants(k.body);
     if (opts.opt_expand_short_loops) k.body = pass.expand_short_loops(k.body, false);
     if (opts.opt_guard_bounds) k.body = pass.guards_to_bounds(k.body);
     if (opts.opt_prefetch_steps) k.body = pass.prefetch_counter_loads(k.body, RangeEnv());
@@ -2679,7 +2734,8 @@ void hip_optimize(Program& p, const Options& opts, NameGen& gen) {
     if (opts.opt_prefetch_steps) k.body = pass.prefetch_selected_rows(k.body, &budget);
     if (opts.opt_reg_cache) pass.reg_cache(&budget);
     if (opts.opt_drop_barriers) pass.drop_barriers();
-    if (opts.opt_noalias_scopes) k.body = pass.noalias_scopes(k.body);
+    k.distinct_pointers.clear();
+    k.body = pass.noalias_scopes(k.body, opts.opt_noalias_scopes);
     pass.mark_read_only();
     k.aligned_params = opts.assume_aligned;
   }

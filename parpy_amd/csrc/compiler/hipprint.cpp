@@ -242,6 +242,7 @@ struct DevicePrinter {
   std::ostringstream os;
   int red_sites = 0;
   std::vector<std::string> lds_decls;
+  std::set<Name> lds_arrays;   // names of the arrays the kernel declares in LDS
 
   explicit DevicePrinter(const Options& o) : opts(o) {}
 
@@ -867,6 +868,24 @@ struct DevicePrinter {
     return false;
   }
 
+  // two different names that cannot stand for the same memory: arrays declared in LDS, pointer parameters that
+  // carry the no-alias promise, local pointers that the alias analysis found never to coincide
+  bool distinct_arrays(const Name& a, const Name& b) const {
+    if (lds_arrays.count(a) && lds_arrays.count(b)) return true;
+    if (!kernel->no_restrict) {
+      bool pa = false, pb = false;
+      for (auto& p : kernel->params) {
+        if (p.ty.k != Type::Pointer) continue;
+        pa = pa || p.id == a;
+        pb = pb || p.id == b;
+      }
+      if (pa && pb) return true;
+    }
+    for (auto& g : kernel->distinct_pointers)
+      if (std::find(g.begin(), g.end(), a) != g.end() && std::find(g.begin(), g.end(), b) != g.end()) return true;
+    return false;
+  }
+
   struct Access { size_t pos; const Expr* e; const Stmt* st; bool store; Name base; Mem mem; E f; int64_t c; bool tracked; };
 
   void plan_packs(const Stmts& ss, size_t lo, size_t hi) {
@@ -894,6 +913,7 @@ struct DevicePrinter {
     }
     auto independent = [&](const Access& a, const Access& b) {
       if (a.mem != b.mem) return true;                                   // LDS and global memory are disjoint
+      if (!(a.base == b.base) && distinct_arrays(a.base, b.base)) return true;
       if (a.tracked && b.tracked && expr_eq(a.f, b.f) && a.c != b.c) return true;   // other elements of the same group
       return false;
     };
@@ -1007,6 +1027,8 @@ struct DevicePrinter {
     narrow_vars.clear();
     reassigned.clear();
     lds_decls.clear();
+    lds_arrays.clear();
+    visit_stmts(k.body, [&](const S& st) { if (st->k == Stmt::LdsDecl) lds_arrays.insert(st->id); });
     pack_loads.clear();
     pack_stores.clear();
     packs.clear();

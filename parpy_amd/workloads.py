@@ -8,7 +8,7 @@ HIP backend -- nothing here calls a hand-written kernel.
 import numpy as np
 
 import parpy_amd as parpy
-from parpy_amd.operators import exp, float32, float64, inf, int32, log, max, sum
+from parpy_amd.operators import exp, float32, float64, inf, int32, log, max, min, sum
 
 
 # ---------------------------------------------------------------- reductions / softmax
@@ -404,6 +404,67 @@ def forward_scaled(hmm, seqs, result, beta1, beta2):
         result[inst] = scale + log(float64(total)) - float64(seqs["lens"][inst]) * hmm["log_emit_scale"]
 
 
+# ---------------------------------------------------------------- HMM forward, reference (16-layer) model, scaled linear space
+@parpy.jit
+def forward_kernel_scaled_step(hmm, seqs, beta1, beta2, inst, t):
+    beta_src = beta2
+    beta_dst = beta1
+    if t & 1:
+        beta_src = beta1
+        beta_dst = beta2
+    o = seqs["data"][inst, t]
+    parpy.label('state')
+    for g in range(hmm["num_states"] // 16):
+        if t < seqs["lens"][inst]:
+            nk = hmm["num_states"] // 16
+            nq = nk // 4
+            q = g % nq
+            lc = g // nq
+            a1 = beta_src[inst, q]
+            a2 = beta_src[inst, nq + q]
+            a3 = beta_src[inst, 2 * nq + q]
+            a4 = beta_src[inst, 3 * nq + q]
+            for l in range(4):
+                layer = 4 * lc + l
+                up = min(layer + 1, 15)
+                for u in range(4):
+                    inflow = (a1 * hmm["ptrans1"][q, u] + a2 * hmm["ptrans1"][nq + q, u] +
+                              a3 * hmm["ptrans1"][2 * nq + q, u] + a4 * hmm["ptrans1"][3 * nq + q, u])
+                    s = hmm["pdur"][layer] * inflow + hmm["pnext"][layer] * beta_src[inst, up * nk + 4 * q + u]
+                    beta_dst[inst, layer * nk + 4 * q + u] = s * hmm["pemit"][o, 4 * q + u]
+
+
+@parpy.jit
+def forward_kernel_scaled(hmm, seqs, result, beta1, beta2):
+    """The forward pass of the reference's 16-layer model (the recurrence of test/test_forward.py:83-160) in
+    linear space with rescaling.  A state is (duration layer, k-mer).  What flows into a k-mer from the four
+    k-mers that precede it (always out of layer 0) is the same for all 16 layers, so one thread computes it once
+    for four neighbouring k-mers and four layers; a layer then adds what comes down from the layer above (from
+    itself in the last layer).  Tables are probabilities: `ptrans1` [4^k, 4], `pdur` [16] (the reference's
+    `trans2`), `pnext` [16] (1 for layers 0..13, 1 - tail for layer 14, tail for the last layer's self loop),
+    `pinit`, and `pemit` [101, 4^k] = emission probabilities times exp(`log_emit_scale`).  The reference's
+    emission tables reach down to 1e-10, so the state vector is divided by its largest element every fourth step.
+    The result is float64, as in `forward_scaled`."""
+    parpy.label('inst')
+    for inst in range(seqs["num_instances"]):
+        o0 = seqs["data"][inst, 0]
+        parpy.label('state')
+        for state in range(hmm["num_states"]):
+            beta1[inst, state] = hmm["pinit"][state] * hmm["pemit"][o0, state % (hmm["num_states"] // 16)]
+        scale = float64(0.0)
+        for t in range(1, seqs["maxlen"]):
+            forward_kernel_scaled_step(hmm, seqs, beta1, beta2, inst, t)
+            if t < seqs["lens"][inst]:
+                if t % 4 == 0:
+                    scale = scale + forward_scaled_renorm(hmm, seqs, beta1, beta2, inst, t)
+        beta = beta1
+        if seqs["lens"][inst] & 1 == 0:
+            beta = beta2
+        parpy.label('state')
+        total = sum(beta[inst, :])
+        result[inst] = scale + log(float64(total)) - float64(seqs["lens"][inst]) * hmm["log_emit_scale"]
+
+
 # ---------------------------------------------------------------- seeded inputs
 SEED = 1234
 
@@ -527,6 +588,20 @@ def with_scaled_tables(hmm):
     probabilities times one constant that makes the largest of them one (`pemit`; `log_emit_scale` is the
     logarithm of that constant, a Python float and so a compile-time constant of the kernel)."""
     out = with_linear_tables(hmm)
+    out["pinit"] = np.exp(hmm["initial_prob"].astype(np.float64)).astype(np.float32)
+    e = hmm["output_prob"].astype(np.float64)
+    out["log_emit_scale"] = float(-e.max())
+    out["pemit"] = np.exp(e + out["log_emit_scale"]).astype(np.float32)
+    return out
+
+
+def with_scaled_reference_tables(hmm):
+    """The reference's 16-layer model with the probability tables `forward_kernel_scaled` reads (see there)."""
+    out = dict(hmm)
+    out["ptrans1"] = np.exp(hmm["trans1"].astype(np.float64)).astype(np.float32)
+    out["pdur"] = np.exp(hmm["trans2"].astype(np.float64)).astype(np.float32)
+    tail = float(np.exp(np.float64(hmm["gamma"])))
+    out["pnext"] = np.array([1.0] * 14 + [1.0 - tail, tail], dtype=np.float32)
     out["pinit"] = np.exp(hmm["initial_prob"].astype(np.float64)).astype(np.float32)
     e = hmm["output_prob"].astype(np.float64)
     out["log_emit_scale"] = float(-e.max())
