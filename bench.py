@@ -1,7 +1,7 @@
 """Benchmark of the compiled hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
-                    [--workload all|hmm7|hmm5|hmm5ref|rowsum|softmax|sddmm|copy] [--form grouped|reference]
+                    [--workload all|hmm7|hmm5|hmm5ref|rowsum|softmax|sddmm|copy] [--form scaled|grouped|reference]
 
 A step is one pass of the compiled function over one batch of seeded synthetic
 input that is already resident in HBM.  The default run (`all`) times the
@@ -18,7 +18,9 @@ tolerance against the fp64 oracle and the `value` of the headline), `grouped`
 (forward_syn4: log space, the four states that share their predecessors updated
 together) and `reference` (forward_syn: log space, one state at a time, the
 structure of the reference's kernel).  The figures of the other forms are in
-the record too.  Results are checked against the oracle outside the timed region.
+the record too.  The reference's own 16-layer model (`hmm5ref`) is timed as its
+kernel (forward_kernel) and in the scaled form (forward_kernel_scaled).  Results
+are checked against the oracle outside the timed region.
 """
 import argparse
 import json
@@ -160,37 +162,67 @@ def bench_hmm(k, args, torch, parpy, W, default_cfg=True):
 def bench_hmm_ref(args, torch, parpy, W, default_cfg=True):
     """The reference's own 5-mer model (16 duration layers x 1024 k-mers = 16384 states) on its 100
     recorded reads, tables from tests/golden: the configuration its benchmark validates
-    (benchmarks/forward.py:481-518).  Results are checked against the expected log-likelihoods."""
+    (benchmarks/forward.py:481-518).  Two statements of the recurrence: the reference's kernel
+    (forward_kernel, log space, checked against the recorded log-likelihoods) and the scaled
+    linear-space form (forward_kernel_scaled, checked against the fp64 oracle)."""
     import numpy as np
+    import oracle
     g = os.path.join(ROOT, "tests", "golden")
     hmm, seqs = W.load_reference_model(os.path.join(g, "hmm_5mer_model.npz"), os.path.join(g, "hmm_signals.npz"))
     want = np.loadtxt(os.path.join(g, "hmm_5mer_expected.txt"), dtype=np.float32)
     S, n = hmm["num_states"], seqs["num_instances"]
-    hd, sd = W.to_device(hmm), W.to_device(seqs)
-    a1 = torch.zeros((n, S), dtype=torch.float32, device="cuda")
-    a2 = torch.zeros_like(a1)
-    res = torch.zeros(n, dtype=torch.float32, device="cuda")
-    nthreads = min(S, args.state_threads)
-    opts = parpy.par({"inst": parpy.threads(n), "state": parpy.threads(nthreads)})
-    _apply_opt_flags(opts, args)
-    fn = lambda: W.forward_kernel(hd, sd, a1, a2, res, opts=opts)
-    timed = lambda: parpy.time_call(W.forward_kernel, hd, sd, a1, a2, res, opts=opts)
-    wall, dev = _events_ms(fn, timed, args.steps, args.warmup, torch)
-    got = res.cpu().numpy()
-    assert np.allclose(got, want, atol=1e-5, rtol=1e-5), float(np.abs(got - want).max())
+    hd, sd = W.to_device(W.with_scaled_reference_tables(hmm)), W.to_device(seqs)
     steps_total = int((seqs["lens"] - 1).sum())
     # per (read, step): alpha read + alpha write (4S each), one emission row of S/16 k-mers, the observation byte
     alg_bytes = (8 * S + 4 * (S // 16) + 1) * steps_total
-    kernel_ms = float(np.median(dev))
+    form = "reference" if args.form == "reference" else "scaled"
+    others = [] if args.single_form else [f for f in ("scaled", "reference") if f != form]
+    sub = np.argsort(seqs["lens"])[:6]
+    want64 = oracle.hmm_ref_forward(hmm, seqs, np.float64, subset=sub)
+    runs = {}
+    for f in [form] + others:
+        a1 = torch.zeros((n, S), dtype=torch.float32, device="cuda")
+        a2 = torch.zeros_like(a1)
+        if f == "scaled":
+            res = torch.zeros(n, dtype=torch.float64, device="cuda")
+            nthreads = min(S // 16, args.state_threads)
+            call = lambda o, res=res, a1=a1, a2=a2: (W.forward_kernel_scaled, (hd, sd, res, a1, a2))
+        else:
+            res = torch.zeros(n, dtype=torch.float32, device="cuda")
+            nthreads = min(S, args.state_threads)
+            call = lambda o, res=res, a1=a1, a2=a2: (W.forward_kernel, (hd, sd, a1, a2, res))
+        opts = parpy.par({"inst": parpy.threads(n), "state": parpy.threads(nthreads)})
+        _apply_opt_flags(opts, args)
+        fun, fargs = call(opts)
+        fn = lambda: fun(*fargs, opts=opts)
+        timed = lambda: parpy.time_call(fun, *fargs, opts=opts)
+        wall, dev = _events_ms(fn, timed, args.steps, args.warmup, torch)
+        got = res.cpu().numpy()
+        if f == "scaled":
+            err = float(np.abs(got[sub] - want64).max())
+            assert np.all(np.isfinite(got)) and err < 1e-4, f"scaled form of the reference model is off by {err}"
+            checked = f"6 shortest reads against the fp64 oracle, max abs error {err:.3g}"
+        else:
+            assert np.allclose(got, want, atol=1e-5, rtol=1e-5), float(np.abs(got - want).max())
+            checked = (f"all {n} reads against the reference's recorded log-likelihoods (atol = rtol = 1e-5), "
+                       f"max abs error {float(np.abs(got - want).max()):.3g}")
+        runs[f] = {"wall": wall, "kernel_ms": float(np.median(dev)), "threads": nthreads, "checked": checked,
+                   "mean": float(got.mean()), "recorded": float(np.abs(got - want).max())}
+    names = {"scaled": "scaled (forward_kernel_scaled)", "reference": "reference (forward_kernel)"}
+    tag = {"scaled": "hmm5ref_scaled", "reference": "hmm5ref"}
+    main = runs[form]
     return {
         "metric": "HMM-forward reference 5-mer model ms/batch + achieved HBM GB/s (% of peak), 1xMI355X",
-        "value": wall, "unit": "ms/batch", "ms_per_step": wall, "higher_is_better": False, "dtype": "f32",
-        "config": {"workload": "hmm_forward_reference_5mer_model", "states": S, "reads": n, "min_len": int(seqs["lens"].min()),
-                   "max_len": int(seqs["lens"].max()), "total_steps": steps_total, "state_threads": nthreads,
-                   "mean_loglik": float(got.mean()),
-                   "checked": f"all {n} reads against the reference's recorded log-likelihoods (atol = rtol = 1e-5), "
-                              f"max abs error {float(np.abs(got - want).max()):.3g}"},
-        "roofline": _hbm_roofline(alg_bytes, kernel_ms, "hmm5ref", default_cfg),
+        "value": main["wall"], "unit": "ms/batch", "ms_per_step": main["wall"], "higher_is_better": False, "dtype": "f32",
+        "config": {"workload": "hmm_forward_reference_5mer_model", "form": names[form],
+                   "result_dtype": "f64" if form == "scaled" else "f32", "states": S, "reads": n,
+                   "min_len": int(seqs["lens"].min()), "max_len": int(seqs["lens"].max()), "total_steps": steps_total,
+                   "state_threads": main["threads"], "mean_loglik": main["mean"], "checked": main["checked"],
+                   "max_abs_distance_to_recorded_f32_values": main["recorded"]},
+        "roofline": _hbm_roofline(alg_bytes, main["kernel_ms"], tag[form], default_cfg),
+        "other_forms": [{"form": names[o], "ms_per_step": runs[o]["wall"], "state_threads": runs[o]["threads"],
+                         "roofline": _hbm_roofline(alg_bytes, runs[o]["kernel_ms"], tag[o], default_cfg),
+                         "checked": runs[o]["checked"]} for o in others],
         "cpu_baseline": None,
         "data": "reference fixtures (tests/golden)",
     }

@@ -471,8 +471,10 @@ struct DevicePrinter {
       case Expr::Convert: return "((" + std::string(elem_ctype(e->ty.sz)) + ")" + paren(pexpr(e->args[0])) + ")";
       case Expr::Index: {
         if (!as_lvalue) {
-          auto pk = pack_loads.find(e.get());
-          if (pk != pack_loads.end()) return pk->second;
+          if (cur_pack_loads) {
+            auto pk = cur_pack_loads->find(e.get());
+            if (pk != cur_pack_loads->end()) return pk->second;
+          }
         }
         // Indexing is in bounds by contract: a variable used as the index of one dimension lies in
         // [0, extent) while this address is computed, which lets gathered indices (loaded from memory,
@@ -727,9 +729,8 @@ struct DevicePrinter {
         std::string rhs = pexpr(s->expr);
         if (s->dst->k == Expr::Var && !s->dst->ty.is_scalar()) rhs = "(" + ctype(s->dst->ty) + ")" + rhs;
         {
-          auto pk = pack_stores.find(s.get());
-          if (pk != pack_stores.end()) {
-            os << ind(n) << packs[pk->second.first].var << "." << "xyzw"[pk->second.second] << " = " << rhs << ";\n";
+          if (cur_pack_store.first >= 0) {
+            os << ind(n) << packs[cur_pack_store.first].var << "." << "xyzw"[cur_pack_store.second] << " = " << rhs << ";\n";
             break;
           }
         }
@@ -823,8 +824,13 @@ struct DevicePrinter {
   // accesses to LDS and to global memory never do.  On LDS this is the difference between four partial-bank
   // accesses and one full-rate one per lane.
   struct Pack { std::string var, decl_ty, addr; bool is_store = false, streamed = false; size_t first = 0, last = 0; const Stmts* owner = nullptr; };
-  std::map<const Expr*, std::string> pack_loads;                   // load expression -> "pk.x"
-  std::map<const Stmt*, std::pair<int, int>> pack_stores;          // store statement -> (pack index, component)
+  // Plans are kept per place (block and position in it), not per node: expression and statement nodes are
+  // shared between the copies that loop expansion and unswitching make.
+  using Place = std::pair<const Stmts*, size_t>;
+  std::map<Place, std::map<const Expr*, std::string>> pack_loads;  // statement -> its load expressions -> "pk.x"
+  std::map<Place, std::pair<int, int>> pack_stores;                // store statement -> (pack index, component)
+  const std::map<const Expr*, std::string>* cur_pack_loads = nullptr;   // of the statement being printed
+  std::pair<int, int> cur_pack_store{-1, -1};
   std::vector<Pack> packs;
   int pack_counter = 0;
 
@@ -988,8 +994,8 @@ struct DevicePrinter {
       static const char* comp = "xyzw";
       for (int c = 0; c < 4; ++c) {
         used.insert(member[c]);
-        if (a0.store) pack_stores[acc[member[c]].st] = {pi, c};
-        else pack_loads[acc[member[c]].e] = pk.var + "." + comp[c];
+        if (a0.store) pack_stores[{&ss, acc[member[c]].pos}] = {pi, c};
+        else pack_loads[{&ss, acc[member[c]].pos}][acc[member[c]].e] = pk.var + "." + comp[c];
       }
     }
   }
@@ -1012,7 +1018,17 @@ struct DevicePrinter {
           if (packs[p].is_store) os << ind(n) << packs[p].decl_ty << " " << packs[p].var << ";\n";
           else os << ind(n) << "const " << packs[p].decl_ty << " " << packs[p].var << " = *" << packs[p].addr << ";\n";
         }
-      pstmt(ss[i], n);
+      {
+        auto saved_loads = cur_pack_loads;
+        auto saved_store = cur_pack_store;
+        auto pl = pack_loads.find({&ss, i});
+        cur_pack_loads = pl == pack_loads.end() ? nullptr : &pl->second;
+        auto ps = pack_stores.find({&ss, i});
+        cur_pack_store = ps == pack_stores.end() ? std::pair<int, int>{-1, -1} : ps->second;
+        pstmt(ss[i], n);
+        cur_pack_loads = saved_loads;
+        cur_pack_store = saved_store;
+      }
       for (size_t p = first_pack; p < packs.size(); ++p)
         if (packs[p].owner == &ss && packs[p].is_store && packs[p].last == i) {
           if (packs[p].streamed) os << ind(n) << "__builtin_nontemporal_store(" << packs[p].var << ", " << packs[p].addr << ");\n";

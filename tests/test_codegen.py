@@ -330,6 +330,46 @@ def test_adjacent_accesses_are_only_packed_when_nothing_they_pass_can_touch_them
     assert "const parpy_vec4<float>" not in s
 
 
+def _reference_format_args(k, n=4, maxlen=30, seed=5):
+    """Random tables in the layout of the reference's 16-layer model, with the probability tables of the scaled form."""
+    rng = np.random.default_rng(seed)
+    nk = 4 ** k
+    hmm = {
+        "trans1": np.log(rng.dirichlet(np.ones(4), size=nk)).astype(np.float32),
+        "trans2": np.log(rng.dirichlet(np.ones(16))).astype(np.float32),
+        "output_prob": np.ascontiguousarray(np.log(rng.dirichlet(np.ones(101), size=nk)).T.astype(np.float32)),
+        "initial_prob": np.concatenate([np.full(nk, -np.log(float(nk))), np.full(15 * nk, -np.inf)]).astype(np.float32),
+        "gamma": np.float32(np.log(0.05)), "synthetic_248": np.float32(np.log1p(-0.05)), "num_states": 16 * nk,
+    }
+    lens = rng.integers(2, maxlen + 1, size=n).astype(np.int64)
+    seqs = {"data": rng.integers(0, 101, size=(n, int(lens.max()))).astype(np.int8), "lens": lens, "maxlen": int(lens.max()), "num_instances": n}
+    b = np.zeros((n, 16 * nk), dtype=np.float32)
+    return [W.with_scaled_reference_tables(hmm), seqs, np.zeros(n, dtype=np.float64), b, b.copy()]
+
+
+def test_scaled_reference_model_step_is_written_out_and_moves_whole_layer_rows():
+    """`forward_kernel_scaled`: local names with constant values (`nk`, `nq`) count as the numbers, the loop over four
+    layers around the loop over four k-mers is written out, and each layer's four neighbouring states are one
+    16-byte LDS load (from the layer above) and one 16-byte LDS store, although the two go through different
+    pointers: the step's source and destination never name the same array."""
+    args = _reference_format_args(4)
+    o = opts_for({'inst': parpy.threads(4), 'state': parpy.threads(256)})
+    s = compiles(parpy.print_compiled(W.forward_kernel_scaled, args, o))
+    step = s[s.index("for (int t_"):]
+    step = step[:step.index("__syncthreads")]
+    assert not re.search(r"for \(int (l|u)_\d+", step) and len(re.findall(r"n[kq]_\d+", step)) == 2   # (only their definitions are left)
+    assert len(re.findall(r"const parpy_vec4<float> pk_\d+ = \*\(__attribute__\(\(address_space\(3\)\)\) const parpy_vec4<float>\*\)&beta_src_\d+\[", step)) == 4
+    assert len(re.findall(r"\*\(__attribute__\(\(address_space\(3\)\)\) parpy_vec4<float>\*\)&beta_dst_\d+\[.*\] = pk_\d+;", step)) == 4
+    # duration and next-layer weights of the thread's four layers and the rows of ptrans1 are loaded once, before the time loop
+    assert "inv_hmm_pdur" in s and "inv_hmm_pnext" in s and "hmm_pdur_" not in step.replace("inv_hmm_pdur", "")
+    # without the step-ahead emission row the four copies of the k-mer loop each load the row: the same expression
+    # nodes in four places, each with its own 16-byte load
+    s1 = compiles(parpy.print_compiled(W.forward_kernel_scaled, args, opts_for({'inst': parpy.threads(4), 'state': parpy.threads(256)}, opt_prefetch_steps=False)))
+    step1 = s1[s1.index("for (int t_"):]
+    step1 = step1[:step1.index("__syncthreads")]
+    assert len(re.findall(r"const parpy_vec4<float> pk_\d+ = \*\(const parpy_vec4<float>\*\)&(parpy_at\()?hmm_pemit_", step1)) == 4
+
+
 def test_noalias_scope_wraps_the_step_body_when_aliases_never_coincide():
     hmm, seqs, args = _hmm_args(4)
     o = opts_for({'inst': parpy.threads(4), 'state': parpy.threads(256)}, opt_noalias_scopes=True)

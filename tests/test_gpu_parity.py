@@ -252,6 +252,65 @@ def test_reference_format_models_with_random_tables(k, threads):
     assert np.all(np.isfinite(want)) and np.allclose(got, want, atol=1e-4, rtol=1e-5), np.abs(got - want).max()
 
 
+def _run_reference_scaled(hmm, seqs, threads, **kw):
+    hd, sd = W.to_device(W.with_scaled_reference_tables(hmm)), W.to_device(seqs)
+    n, S = seqs["num_instances"], hmm["num_states"]
+    b1 = torch.zeros((n, S), dtype=torch.float32, device="cuda")
+    b2 = torch.zeros_like(b1)
+    res = torch.zeros(n, dtype=torch.float64, device="cuda")
+    W.forward_kernel_scaled(hd, sd, res, b1, b2, opts=opts_for({'inst': parpy.threads(n), 'state': parpy.threads(threads)}, **kw))
+    return res.cpu().numpy()
+
+
+@pytest.mark.parametrize("threads", [64, 256])
+def test_reference_model_scaled_form_3mer_golden(golden_dir, threads):
+    """The reference's 3-mer model and reads in linear space with rescaling: within 1e-4 of the fp64 oracle on every
+    read, and as close to the recorded (single precision, log space) likelihoods as those are to the fp64 oracle."""
+    hmm, seqs, exp = _golden(golden_dir, 3)
+    got = _run_reference_scaled(hmm, seqs, threads)
+    want = oracle.hmm_ref_forward(hmm, seqs, np.float64)
+    assert np.abs(got - want).max() < 1e-4, np.abs(got - want).max()
+    assert np.all(np.abs(got - exp) <= np.abs(exp - want) + 1e-3)
+
+
+def test_reference_model_scaled_form_5mer_golden(golden_dir):
+    """16384 states, 100 reads of 2779..8885 samples, emission probabilities down to 1e-10: every fourth read against
+    the fp64 oracle (the recorded single-precision values are up to 0.26 away from it), all reads against the
+    recorded values at the tolerance the reference's test allows them."""
+    hmm, seqs, exp = _golden(golden_dir, 5)
+    got = _run_reference_scaled(hmm, seqs, 1024)
+    sub = list(range(0, seqs["num_instances"], 4))
+    want = oracle.hmm_ref_forward(hmm, seqs, np.float64, subset=sub)
+    assert np.abs(got[sub] - want).max() < 1e-4, np.abs(got[sub] - want).max()
+    assert np.allclose(got, exp, atol=1e-5, rtol=2e-5), np.abs(got - exp).max()
+
+
+@pytest.mark.parametrize("k,threads", [(1, 64), (2, 64), (3, 64), (3, 32), (4, 256), (4, 1024), (5, 512)])
+def test_reference_format_models_with_random_tables_scaled_form(k, threads):
+    hmm, seqs = _random_reference_model(k, n_reads=4, max_len=37, seed=100 * k + threads)
+    got = _run_reference_scaled(hmm, seqs, threads)
+    want = oracle.hmm_ref_forward(hmm, seqs, np.float64)
+    assert np.all(np.isfinite(want)) and np.abs(got - want).max() < 1e-4, np.abs(got - want).max()
+
+
+@pytest.mark.parametrize("flags", [{"opt_pack_accesses": False}, {"opt_expand_short_loops": False}, {"opt_prefetch_steps": False},
+                                   {"opt_lds_rows": False}, {"opt_guard_bounds": False}, {"opt_hoist_invariant": False},
+                                   {"opt_vectorize": False, "opt_reg_cache": False}], ids=lambda f: "+".join(f))
+def test_reference_model_scaled_form_each_pass_preserves_results(golden_dir, flags):
+    hmm, seqs, exp = _golden(golden_dir, 3)
+    got = _run_reference_scaled(hmm, seqs, 64, **flags)
+    want = oracle.hmm_ref_forward(hmm, seqs, np.float64)
+    assert np.abs(got - want).max() < 1e-4, (flags, np.abs(got - want).max())
+
+
+def test_reference_model_scaled_form_with_state_vectors_larger_than_lds():
+    """65536 states: the state vectors stay in global memory, one workgroup per read."""
+    hmm, seqs = _random_reference_model(6, n_reads=3, max_len=12, seed=11)
+    got = _run_reference_scaled(hmm, seqs, 1024)
+    want = oracle.hmm_ref_forward(hmm, seqs, np.float64)
+    assert np.all(np.isfinite(want)) and np.abs(got - want).max() < 1e-4, np.abs(got - want).max()
+
+
 def _run_synthetic(hmm, seqs, threads, **kw):
     hd, sd = W.to_device(hmm), W.to_device(seqs)
     n, S = seqs["num_instances"], hmm["num_states"]
