@@ -47,7 +47,7 @@ VALU_NS = {"full": 1.17, "trans": 3.76}
 HMM_VALU_MIX = {
     "reference": {"full": 24.0, "trans": 6.0},
     "grouped": {"full": 14.2, "trans": 3.0},
-    "scaled": {"full": 7.5, "trans": 0.0},
+    "scaled": {"full": 8.4, "trans": 0.0},
 }
 HMM_FORMS = {"scaled": "forward_scaled", "grouped": "forward_syn4", "reference": "forward_syn"}
 

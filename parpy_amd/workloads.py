@@ -341,7 +341,7 @@ def forward_syn4(hmm, seqs, result, alpha1, alpha2):
 
 # ---------------------------------------------------------------- HMM forward, synthetic model, scaled linear space
 @parpy.jit
-def forward_scaled_step(hmm, seqs, beta1, beta2, inst, t):
+def forward_scaled_step(hmm, seqs, beta1, beta2, inst, t, r):
     beta_src = beta2
     beta_dst = beta1
     if t & 1:
@@ -360,19 +360,17 @@ def forward_scaled_step(hmm, seqs, beta1, beta2, inst, t):
                 s = (a1 * hmm["ptrans1"][q, u] + a2 * hmm["ptrans1"][nq + q, u] +
                      a3 * hmm["ptrans1"][2 * nq + q, u] + a4 * hmm["ptrans1"][3 * nq + q, u] +
                      beta_src[inst, 4 * q + u] * hmm["pstay"][4 * q + u])
-                beta_dst[inst, 4 * q + u] = s * hmm["pemit"][o, 4 * q + u]
+                beta_dst[inst, 4 * q + u] = (s * r) * hmm["pemit"][o, 4 * q + u]
 
 
 @parpy.jit
-def forward_scaled_renorm(hmm, seqs, beta1, beta2, inst, t):
+def forward_scaled_top(hmm, seqs, beta1, beta2, inst, t):
     beta = beta1
     if t & 1:
         beta = beta2
     parpy.label('state')
     top = max(beta[inst, :])
-    parpy.label('state')
-    beta[inst, :] = beta[inst, :] * (float32(1.0) / top)
-    return log(float64(top))
+    return top
 
 
 @parpy.jit
@@ -380,9 +378,13 @@ def forward_scaled(hmm, seqs, result, beta1, beta2):
     """The forward pass of the synthetic model in linear space with rescaling (the classical alternative to
     log space): beta[s] holds the probability alpha[s] times a running scale whose logarithm is kept in
     float64.  Tables are probabilities: `ptrans1`, `pstay`, `pinit`, and `pemit` = emission probabilities
-    times the constant exp(`log_emit_scale`) that makes the largest of them one.  A step is five multiply-adds
-    and one multiplication per state, no exponential and no logarithm; every eighth step the state vector is
-    divided by its largest element.  The result is float64:
+    times the constant exp(`log_emit_scale`) that makes the largest of them one.  A step is one multiplication
+    and four multiply-adds per state for the sum over its predecessors and itself and two multiplications (by the
+    divisor `r` and by the emission), no exponential and no logarithm.  Every eighth step the largest element of
+    the new state vector is looked up; the vector itself is left alone and the next step divides what it
+    produces by that element (the step is linear, so this is the same as dividing its input, without a second
+    pass over the vector).  The divisors are collected as a float64 product whose logarithm is taken every 64
+    steps.  The result is float64:
     log-likelihood = log(sum of the final vector) + sum of log(divisors) - len * log_emit_scale."""
     parpy.label('inst')
     for inst in range(seqs["num_instances"]):
@@ -391,22 +393,30 @@ def forward_scaled(hmm, seqs, result, beta1, beta2):
         for state in range(hmm["num_states"]):
             beta1[inst, state] = hmm["pinit"][state] * hmm["pemit"][o0, state]
         scale = float64(0.0)
+        tops = float64(1.0)
+        r = float32(1.0)
         for t in range(1, seqs["maxlen"]):
-            forward_scaled_step(hmm, seqs, beta1, beta2, inst, t)
+            forward_scaled_step(hmm, seqs, beta1, beta2, inst, t, r)
             if t < seqs["lens"][inst]:
+                r = float32(1.0)
                 if t % 8 == 0:
-                    scale = scale + forward_scaled_renorm(hmm, seqs, beta1, beta2, inst, t)
+                    top = forward_scaled_top(hmm, seqs, beta1, beta2, inst, t)
+                    r = float32(1.0) / top
+                    tops = tops * float64(top)
+                    if t % 64 == 0:
+                        scale = scale + log(tops)
+                        tops = float64(1.0)
         beta = beta1
         if seqs["lens"][inst] & 1 == 0:
             beta = beta2
         parpy.label('state')
         total = sum(beta[inst, :])
-        result[inst] = scale + log(float64(total)) - float64(seqs["lens"][inst]) * hmm["log_emit_scale"]
+        result[inst] = scale + log(float64(total) * float64(r) * tops) - float64(seqs["lens"][inst]) * hmm["log_emit_scale"]
 
 
 # ---------------------------------------------------------------- HMM forward, reference (16-layer) model, scaled linear space
 @parpy.jit
-def forward_kernel_scaled_step(hmm, seqs, beta1, beta2, inst, t):
+def forward_kernel_scaled_step(hmm, seqs, beta1, beta2, inst, t, r):
     beta_src = beta2
     beta_dst = beta1
     if t & 1:
@@ -431,7 +441,7 @@ def forward_kernel_scaled_step(hmm, seqs, beta1, beta2, inst, t):
                     inflow = (a1 * hmm["ptrans1"][q, u] + a2 * hmm["ptrans1"][nq + q, u] +
                               a3 * hmm["ptrans1"][2 * nq + q, u] + a4 * hmm["ptrans1"][3 * nq + q, u])
                     s = hmm["pdur"][layer] * inflow + hmm["pnext"][layer] * beta_src[inst, up * nk + 4 * q + u]
-                    beta_dst[inst, layer * nk + 4 * q + u] = s * hmm["pemit"][o, 4 * q + u]
+                    beta_dst[inst, layer * nk + 4 * q + u] = (s * r) * hmm["pemit"][o, 4 * q + u]
 
 
 @parpy.jit
@@ -443,8 +453,9 @@ def forward_kernel_scaled(hmm, seqs, result, beta1, beta2):
     itself in the last layer).  Tables are probabilities: `ptrans1` [4^k, 4], `pdur` [16] (the reference's
     `trans2`), `pnext` [16] (1 for layers 0..13, 1 - tail for layer 14, tail for the last layer's self loop),
     `pinit`, and `pemit` [101, 4^k] = emission probabilities times exp(`log_emit_scale`).  The reference's
-    emission tables reach down to 1e-10, so the state vector is divided by its largest element every fourth step.
-    The result is float64, as in `forward_scaled`."""
+    emission tables reach down to 1e-10, so the divisor is renewed every fourth step (in the way described at
+    `forward_scaled`: the largest element is looked up, the next step divides by it) and the logarithm of the
+    collected divisors is taken every 32 steps.  The result is float64, as in `forward_scaled`."""
     parpy.label('inst')
     for inst in range(seqs["num_instances"]):
         o0 = seqs["data"][inst, 0]
@@ -452,17 +463,25 @@ def forward_kernel_scaled(hmm, seqs, result, beta1, beta2):
         for state in range(hmm["num_states"]):
             beta1[inst, state] = hmm["pinit"][state] * hmm["pemit"][o0, state % (hmm["num_states"] // 16)]
         scale = float64(0.0)
+        tops = float64(1.0)
+        r = float32(1.0)
         for t in range(1, seqs["maxlen"]):
-            forward_kernel_scaled_step(hmm, seqs, beta1, beta2, inst, t)
+            forward_kernel_scaled_step(hmm, seqs, beta1, beta2, inst, t, r)
             if t < seqs["lens"][inst]:
+                r = float32(1.0)
                 if t % 4 == 0:
-                    scale = scale + forward_scaled_renorm(hmm, seqs, beta1, beta2, inst, t)
+                    top = forward_scaled_top(hmm, seqs, beta1, beta2, inst, t)
+                    r = float32(1.0) / top
+                    tops = tops * float64(top)
+                    if t % 32 == 0:
+                        scale = scale + log(tops)
+                        tops = float64(1.0)
         beta = beta1
         if seqs["lens"][inst] & 1 == 0:
             beta = beta2
         parpy.label('state')
         total = sum(beta[inst, :])
-        result[inst] = scale + log(float64(total)) - float64(seqs["lens"][inst]) * hmm["log_emit_scale"]
+        result[inst] = scale + log(float64(total) * float64(r) * tops) - float64(seqs["lens"][inst]) * hmm["log_emit_scale"]
 
 
 # ---------------------------------------------------------------- seeded inputs
