@@ -10,6 +10,7 @@ like the reference does (src/utils/err.rs:79-87, src/utils/info.rs:90-121).
 import ctypes
 import linecache
 import os
+import warnings
 import pathlib
 import subprocess
 
@@ -24,11 +25,15 @@ SOURCES = ["ast.cpp", "front.cpp", "constfold.cpp", "specialize.cpp", "lower.cpp
 _lib = None
 
 
+def _stale():
+    deps = [CSRC / s for s in SOURCES] + list(CSRC.glob("*.hpp")) + [pathlib.Path(__file__).parent.parent / "include" / "parpy_hipc.h"]
+    return any(os.path.getmtime(LIB_PATH) < os.path.getmtime(d) for d in deps if d.exists())
+
+
 def build_library(force=False):
     """Compile the compiler core with g++ (no GPU toolchain needed)."""
     srcs = [CSRC / s for s in SOURCES]
-    deps = srcs + list(CSRC.glob("*.hpp")) + [pathlib.Path(__file__).parent.parent / "include" / "parpy_hipc.h"]
-    if not force and LIB_PATH.exists() and all(os.path.getmtime(LIB_PATH) >= os.path.getmtime(d) for d in deps):
+    if not force and LIB_PATH.exists() and not _stale():
         return LIB_PATH
     cmd = ["g++", "-std=c++17", "-O2", "-fPIC", "-shared", "-Wall", "-Wno-sign-compare",
            "-o", str(LIB_PATH)] + [str(s) for s in srcs]
@@ -42,8 +47,11 @@ def _load():
     global _lib
     if _lib is not None:
         return _lib
-    if not LIB_PATH.exists():
+    # (as for the runtime library: what is built is loaded; a library older than its sources is rebuilt on request)
+    if not LIB_PATH.exists() or os.environ.get("PARPY_AMD_REBUILD") == "1":
         build_library()
+    elif _stale():
+        warnings.warn(f"{LIB_PATH.name} is older than its sources: run __graft_entry__.build() or set PARPY_AMD_REBUILD=1", RuntimeWarning)
     lib = ctypes.CDLL(str(LIB_PATH))
     vp, cp, i32 = ctypes.c_void_p, ctypes.c_char_p, ctypes.c_int32
     lib.parpy_hipc_parse.argtypes = [cp, ctypes.POINTER(cp), ctypes.POINTER(vp), i32, ctypes.POINTER(vp)]

@@ -8,6 +8,7 @@ file is present.
 """
 import ctypes
 import os
+import warnings
 import pathlib
 import subprocess
 
@@ -21,14 +22,22 @@ HIPCC_FLAGS = ["-O2", "-fPIC", "-shared", "-std=c++17", "--offload-arch=gfx950",
 libs = {}
 
 
+def _older_than(lib, deps):
+    return any(os.path.getmtime(lib) < os.path.getmtime(d) for d in deps if d.exists())
+
+
+def _runtime_deps():
+    return [PARPY_NATIVE_PATH / "parpy_hip.cpp", pathlib.Path(__file__).parent / "csrc" / "compiler" / "sexpr.hpp",
+            pathlib.Path(__file__).parent.parent / "include" / "parpy_hip.h"]
+
+
 def build_library(force=False):
     """Compile csrc/runtime/parpy_hip.cpp with hipcc for gfx950 (host code plus the device scratch array;
     cross-compiles without a GPU)."""
     src = PARPY_NATIVE_PATH / "parpy_hip.cpp"
-    deps = [src, pathlib.Path(__file__).parent / "csrc" / "compiler" / "sexpr.hpp",
-            pathlib.Path(__file__).parent.parent / "include" / "parpy_hip.h"]
+    deps = _runtime_deps()
     lib = PARPY_HIP_BASE_LIB_PATH
-    if not force and lib.exists() and all(os.path.getmtime(lib) >= os.path.getmtime(d) for d in deps):
+    if not force and lib.exists() and not _older_than(lib, deps):
         return lib
     cmd = ["hipcc"] + HIPCC_FLAGS + ["-o", str(lib), str(src), "-lhiprtc"]
     r = subprocess.run(cmd, capture_output=True, text=True)
@@ -88,8 +97,13 @@ def init_library(libpath):
 def load_hip_runtime_lib():
     """Load the runtime library without requiring a GPU (hiprtc compilation works on any host)."""
     if "hip-nogpu" not in libs:
-        if not PARPY_HIP_BASE_LIB_PATH.exists():
+        # A library that is there is loaded as it is (a GPU machine runs what was built beforehand); one that is
+        # older than its sources is rebuilt only on request and otherwise named in a warning.
+        if not PARPY_HIP_BASE_LIB_PATH.exists() or os.environ.get("PARPY_AMD_REBUILD") == "1":
             build_library()
+        elif _older_than(PARPY_HIP_BASE_LIB_PATH, _runtime_deps()):
+            warnings.warn(f"{PARPY_HIP_BASE_LIB_PATH.name} is older than its sources: run __graft_entry__.build() "
+                          "or set PARPY_AMD_REBUILD=1", RuntimeWarning)
         libs["hip-nogpu"] = init_library(PARPY_HIP_BASE_LIB_PATH)
     return libs["hip-nogpu"]
 

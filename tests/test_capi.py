@@ -54,3 +54,19 @@ def test_plan_rejects_malformed_text_and_wrong_arity():
     assert b"expects 1 pointer arguments" in lib.parpy_get_error_message()
     assert lib.parpy_hip_plan_run(plan, args, 1) != 0   # no module loaded: refuses to run
     assert lib.parpy_hip_plan_destroy(plan) == 0
+
+
+def test_a_library_older_than_its_sources_is_loaded_with_a_warning_and_rebuilt_only_on_request(monkeypatch):
+    from parpy_amd import runtime
+    built = []
+    monkeypatch.setattr(runtime, "_older_than", lambda lib, deps: True)
+    monkeypatch.setattr(runtime, "build_library", lambda force=False: built.append(force))
+    monkeypatch.delitem(runtime.libs, "hip-nogpu", raising=False)
+    monkeypatch.delenv("PARPY_AMD_REBUILD", raising=False)
+    with pytest.warns(RuntimeWarning, match="older than its sources"):
+        assert runtime.load_hip_runtime_lib() is not None
+    assert built == []
+    monkeypatch.delitem(runtime.libs, "hip-nogpu", raising=False)
+    monkeypatch.setenv("PARPY_AMD_REBUILD", "1")
+    runtime.load_hip_runtime_lib()
+    assert built == [False]
