@@ -387,6 +387,7 @@ struct Options {  // src/option.rs:14-108
   bool opt_guard_bounds = true;       // `for t: if t < X: work` with X fixed and uniform runs to min(hi, X) without the test
   bool opt_prefetch_steps = true;     // loads indexed by the counter of a barrier-stepped loop are issued one step ahead
   bool opt_pack_accesses = true;      // four adjacent 4-byte accesses of one iteration become one 16-byte access
+  bool opt_share_iterations = true;   // what all iterations of one thread have in common is evaluated once per thread
   bool opt_expand_short_loops = true; // counted loops of <= 8 iterations inside a parallel iteration are expanded in place
   int64_t reg_budget = 0;     // 32-bit registers per thread the caching passes may claim (0 = by block size)
   bool assume_aligned = true;  // array arguments are at least 16-byte aligned

@@ -1613,6 +1613,220 @@ struct Pass {
     return out;
   }
 
+  // ================================================================ what the iterations of one thread share
+  // A parallel loop of `per * N` iterations on N threads gives thread g the iterations g, g + N, ..., g + (per-1) N.
+  // When N is a multiple of what the body divides by, much of the body is the same in all of them: with one thread
+  // per k-mer of a 16-layer model (`state = g + layer * N`) the four predecessors `(state // 4) % (N // 4)`, their
+  // table rows, their scores and the emission `output_prob[o, state % N]` depend on g alone.  The loop variable is
+  // replaced by `g + k * N`, quotients and remainders of such sums are taken apart where the constants divide
+  // ((a + k * N) // c = a // c + k * (N // c), (a + k * N) % c = a % c for c | N and a, k >= 0; a // c = 0 and
+  // a % c = a where the range of a says so), and the largest subexpressions that are free of k -- loads
+  // included -- are evaluated once per thread in front of the counted loop (the statements kept in `els` of the
+  // loop, printed before it).  A load may move there because the iterations of a parallel loop do not depend on
+  // each other: what one reads no other writes.  On top of that the array must not be stored to by name in the
+  // body, and must be either never written by the kernel or known to differ from every array the body stores to
+  // (pointer parameters carry the no-alias promise; local pointers that never coincide).
+  struct OwnIterations {
+    Pass& p;
+    Name gname, kname;
+    int64_t N = 0, per = 0;
+    RangeEnv env;
+    std::set<Name> variant;            // names whose value changes with k
+    std::set<Name> stored;             // arrays the body stores to
+    std::set<Name> never_written;      // parameters the kernel only reads
+    Stmts pre;
+    ElemSize isz;
+
+    bool divides_all(const E& e, int64_t c) const {   // e is a multiple of c for every value of its variables
+      if (e->k == Expr::Int) return e->iv % c == 0;
+      if (e->k == Expr::Convert) return divides_all(e->args[0], c);
+      if (e->k != Expr::BinOpE) return false;
+      if (e->bop == BinOp::Mul)
+        return (e->args[0]->k == Expr::Int && e->args[0]->iv % c == 0) || (e->args[1]->k == Expr::Int && e->args[1]->iv % c == 0);
+      if (e->bop == BinOp::Add) return divides_all(e->args[0], c) && divides_all(e->args[1], c);
+      return false;
+    }
+    bool non_negative(const E& e) const {
+      Interval r = expr_range(e, env);
+      return r.known && r.lo >= 0;
+    }
+    E divide(const E& e, int64_t c) const {            // e / c for e with divides_all(e, c)
+      if (e->k == Expr::Int) return mk_int(e->iv / c, e->ty.sz, e->i);
+      if (e->k == Expr::Convert) return mk_convert(divide(e->args[0], c), e->ty.sz);
+      if (e->bop == BinOp::Mul) {
+        if (e->args[0]->k == Expr::Int && e->args[0]->iv % c == 0)
+          return fold_expr(mk_binop(BinOp::Mul, mk_int(e->args[0]->iv / c, e->args[0]->ty.sz), e->args[1], e->ty, e->i));
+        return fold_expr(mk_binop(BinOp::Mul, e->args[0], mk_int(e->args[1]->iv / c, e->args[1]->ty.sz), e->ty, e->i));
+      }
+      return fold_expr(mk_binop(BinOp::Add, divide(e->args[0], c), divide(e->args[1], c), e->ty, e->i));
+    }
+    E simplify(const E& e0) const {
+      return rewrite_expr(e0, [&](const E& e) -> E {
+        if (e->k != Expr::BinOpE || !e->ty.is_scalar() || !is_int(e->ty.sz)) return e;
+        bool div = e->bop == BinOp::FloorDiv || e->bop == BinOp::Div, rem = e->bop == BinOp::Rem;
+        if (!(div || rem) || e->args[1]->k != Expr::Int || e->args[1]->iv <= 0) return e;
+        int64_t c = e->args[1]->iv;
+        const E& a = e->args[0];
+        Interval r = expr_range(a, env);
+        if (r.known && r.lo >= 0 && r.hi < c) return div ? mk_int(0, e->ty.sz, e->i) : a;
+        if (a->k == Expr::BinOpE && a->bop == BinOp::Add && a->ty == e->ty) {
+          for (int side = 0; side < 2; ++side) {
+            const E &m = a->args[side], &rest = a->args[1 - side];
+            if (!divides_all(m, c) || !non_negative(m) || !non_negative(rest)) continue;
+            if (rem) return simplify(mk_binop(BinOp::Rem, rest, e->args[1], e->ty, e->i));
+            return fold_expr(mk_binop(BinOp::Add, simplify(mk_binop(e->bop, rest, e->args[1], e->ty, e->i)), divide(m, c), e->ty, e->i));
+          }
+        }
+        return e;
+      });
+    }
+    bool load_may_move(const E& x) const {
+      if (x->args[0]->k != Expr::Var) return false;
+      const Name& b = x->args[0]->name;
+      if (stored.count(b)) return false;
+      if (never_written.count(b)) return true;
+      for (auto& sb : stored)
+        if (!p.distinct_names(b, sb)) return false;
+      return true;
+    }
+    bool shared(const E& e) const {                    // the same in every iteration of the thread
+      bool ok = true;
+      visit_exprs(e, [&](const E& x) {
+        if (x->k == Expr::Var && (x->name == kname || variant.count(x->name))) ok = false;
+        if (x->k == Expr::Index && !load_may_move(x)) ok = false;
+        if (x->k == Expr::Call || x->k == Expr::Raw || x->k == Expr::RegElem || x->k == Expr::AddrOf) ok = false;
+      });
+      return ok;
+    }
+    static bool worth(const E& e) {
+      bool w = false;
+      visit_exprs(e, [&](const E& x) {
+        if (x->k == Expr::Index) w = true;
+        if (x->k == Expr::BinOpE && (x->bop == BinOp::FloorDiv || x->bop == BinOp::Div || x->bop == BinOp::Rem)) w = true;
+      });
+      return w;
+    }
+    E lift(const E& e) {
+      if (!e) return e;
+      if (e->ty.is_scalar() && shared(e) && worth(e)) {
+        for (auto& d : pre)
+          if (d->k == Stmt::Def && d->ty == e->ty && expr_eq(d->expr, e)) return mk_var(d->id, d->ty, e->i);
+        Name n = p.gen.fresh("own");
+        pre.push_back(mk_def(n, e->ty, e, e->i));
+        Interval r = expr_range(e, env);
+        if (r.known) env[n] = r;
+        return mk_var(n, e->ty, e->i);
+      }
+      // what a selection or a short-circuit operator may skip stays where it is (a test can guard an index)
+      if (e->k == Expr::IfExpr || (e->k == Expr::BinOpE && (e->bop == BinOp::And || e->bop == BinOp::Or))) {
+        auto n = std::make_shared<Expr>(*e);
+        n->args[0] = lift(e->args[0]);
+        return n;
+      }
+      return map_children(e, [&](const E& c) { return lift(c); });
+    }
+  };
+
+  bool distinct_names(const Name& a, const Name& b) const {
+    if (a == b) return false;
+    bool pa = false, pb = false;
+    for (auto& q : k.params) {
+      if (!q.ty.is_pointer()) continue;
+      pa = pa || q.id == a;
+      pb = pb || q.id == b;
+    }
+    if (pa && pb && !k.no_restrict) return true;
+    for (auto& g : k.distinct_pointers)
+      if (std::find(g.begin(), g.end(), a) != g.end() && std::find(g.begin(), g.end(), b) != g.end()) return true;
+    return false;
+  }
+
+  Stmts share_own_iterations(const Stmts& ss) {
+    Stmts out;
+    for (auto& s : ss) {
+      bool mapped = s->k == Stmt::For && (s->map.k == GpuMap::Thread || s->map.k == GpuMap::ThreadBlock);
+      int64_t extent = mapped ? const_extent(s) : -1;
+      bool fits = mapped && s->els.empty() && s->step == 1 && extent > 0 && s->lo->iv == 0 && extent % s->map.n == 0 &&
+                  extent / s->map.n > 1 && (s->map.k == GpuMap::Thread || s->map.n % s->map.tpb == 0) && !s->unroll;
+      if (fits) {
+        for (auto& c : s->body)
+          if (c->k != Stmt::Def && c->k != Stmt::Assign) fits = false;
+        visit_stmts(s->body, [&](const S& c) {
+          visit_stmt_exprs(c, [&](const E& x) { if (x->k == Expr::RegElem || x->k == Expr::AddrOf) fits = false; });
+        });
+      }
+      if (!fits) {
+        auto r = clone(s);
+        r->body = share_own_iterations(s->body);
+        if (s->k != Stmt::For) r->els = share_own_iterations(s->els);
+        out.push_back(r);
+        continue;
+      }
+      OwnIterations oi{*this};
+      oi.isz = isz;
+      oi.N = s->map.n;
+      oi.per = extent / s->map.n;
+      oi.gname = Name{s->id.str() + "_g", 0};
+      oi.kname = Name{s->id.str() + "_k", 0};
+      Type ity = s->lo->ty;
+      Interval gr, kr;
+      gr.known = kr.known = true;
+      gr.lo = kr.lo = 0;
+      gr.hi = oi.N - 1;
+      kr.hi = oi.per - 1;
+      oi.env[oi.gname] = gr;
+      oi.env[oi.kname] = kr;
+      std::set<Name> written = written_arrays();
+      for (auto& q : k.params)
+        if (q.ty.is_pointer() && !written.count(q.id)) oi.never_written.insert(q.id);
+      std::set<Name> defined, reassigned;
+      bool ok = true;
+      for (auto& c : s->body) {
+        if (c->k == Stmt::Def) defined.insert(c->id);
+        if (c->k == Stmt::Assign && c->dst->k == Expr::Var) {
+          if (!defined.count(c->dst->name)) ok = false;   // a value that lives across iterations: not ours to move
+          reassigned.insert(c->dst->name);
+        }
+        if (c->k == Stmt::Assign && c->dst->k == Expr::Index) {
+          if (c->dst->args[0]->k == Expr::Var) oi.stored.insert(c->dst->args[0]->name); else ok = false;
+        }
+      }
+      if (!ok) { out.push_back(s); continue; }
+      oi.variant = reassigned;
+      E sum = mk_binop(BinOp::Add, mk_var(oi.gname, ity), mk_binop(BinOp::Mul, mk_var(oi.kname, ity), mk_int(oi.N, ity.sz), ity), ity);
+      std::map<Name, E> sub;
+      sub[s->id] = sum;
+      Stmts body;
+      for (auto& c : s->body) {
+        auto r = clone(c);
+        E e = oi.simplify(fold_expr(subst_vars(c->expr, sub)));
+        if (c->k == Stmt::Def && c->ty.is_scalar() && !reassigned.count(c->id) && oi.shared(e)) {
+          // the whole definition is the same for all iterations of the thread
+          r->expr = e;
+          oi.pre.push_back(r);
+          Interval rg = expr_range(e, oi.env);
+          if (rg.known) oi.env[c->id] = rg;
+          continue;
+        }
+        r->expr = oi.lift(e);
+        if (c->k == Stmt::Def) {
+          oi.variant.insert(c->id);
+          Interval rg = expr_range(r->expr, oi.env);
+          if (rg.known && !reassigned.count(c->id)) oi.env[c->id] = rg;
+        } else if (c->dst->k == Expr::Index) {
+          r->dst = map_children(c->dst, [&](const E& x) { return oi.lift(oi.simplify(fold_expr(subst_vars(x, sub)))); });
+        }
+        body.push_back(r);
+      }
+      if (oi.pre.empty()) { out.push_back(s); continue; }
+      auto ns = clone(s);
+      ns->body = body;
+      ns->els = oi.pre;
+      out.push_back(ns);
+    }
+    return out;
+  }
+
   // ================================================================ register caching across parallel loops
   // Consecutive thread-mapped loops with the same iteration structure give each
   // thread the same elements every time.  An array that is only ever accessed
@@ -2010,13 +2224,14 @@ struct Pass {
     std::vector<E> params;
     for (auto& n : order)
       if (types.count(n) && types[n].k == Type::Pointer) params.push_back(mk_var(n, types[n]));
-    if (params.size() < 2) return cur;
     if (!wrap) {
       std::vector<Name> group;
-      for (auto& e : params) group.push_back(e->name);
-      k.distinct_pointers.push_back(group);
+      for (auto& n : order)
+        if (types.count(n)) group.push_back(n);
+      if (group.size() >= 2) k.distinct_pointers.push_back(group);
       return cur;
     }
+    if (params.size() < 2) return cur;
     auto scope = std::make_shared<Stmt>();
     scope->k = Stmt::Scope;
     scope->args = params;
@@ -2733,6 +2948,11 @@ void hip_optimize(Program& p, const Options& opts, NameGen& gen) {
     if (opts.opt_hoist_invariant) k.body = pass.hoist_invariant(k.body, &budget, false);
     if (opts.opt_prefetch_steps) k.body = pass.prefetch_selected_rows(k.body, &budget);
     if (opts.opt_reg_cache) pass.reg_cache(&budget);
+    if (opts.opt_share_iterations) {
+      k.distinct_pointers.clear();
+      pass.noalias_scopes(k.body, false);
+      k.body = pass.share_own_iterations(k.body);
+    }
     if (opts.opt_drop_barriers) pass.drop_barriers();
     k.distinct_pointers.clear();
     k.body = pass.noalias_scopes(k.body, opts.opt_noalias_scopes);

@@ -667,6 +667,21 @@ struct DevicePrinter {
         ranges[Name{k, 0}] = kr;
         narrow_vars.insert(Name{k, 0});
       }
+      // what the thread's iterations have in common (kept in `els` by the pass that finds it) comes first, in
+      // terms of the thread's first iteration `<v>_g`
+      bool shared_first = !s->els.empty();
+      if (shared_first) {
+        os << ind(n) << "{\n";
+        n += 2;
+        Interval gr;
+        gr.known = true;
+        gr.lo = 0;
+        gr.hi = N - 1;
+        ranges[Name{v + "_g", 0}] = gr;
+        narrow_vars.insert(Name{v + "_g", 0});
+        os << ind(n) << "int " << v << "_g = " << idx << ";\n";
+        pstmts(s->els, n);
+      }
       if (s->unroll) {
         os << ind(n) << "#pragma unroll\n";
       } else {
@@ -679,7 +694,7 @@ struct DevicePrinter {
         os << ind(n) << "#pragma unroll " << (threads >= 1024 ? 2 : 4) << "\n";
       }
       os << ind(n) << "for (int " << k << " = 0; " << k << " < " << per << "; ++" << k << ") {\n";
-      os << ind(n + 2) << vty << " " << v << " = " << init("(" + idx + " + " + k + " * " + std::to_string(N) + ")") << ";\n";
+      os << ind(n + 2) << vty << " " << v << " = " << init("(" + (shared_first ? v + "_g" : idx) + " + " + k + " * " + std::to_string(N) + ")") << ";\n";
       if (ragged) {
         os << ind(n + 2) << "if (" << v << cmp << his << ") {\n";
         pstmts(s->body, n + 4);
@@ -688,6 +703,10 @@ struct DevicePrinter {
         pstmts(s->body, n + 2);
       }
       os << ind(n) << "}\n";
+      if (shared_first) {
+        n -= 2;
+        os << ind(n) << "}\n";
+      }
       return;
     }
     std::string cond = v + cmp + his;

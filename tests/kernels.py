@@ -239,3 +239,11 @@ def forward_in_pieces(hmm, seqs, alpha1, alpha2, result):
         for t in range(1, seqs["maxlen"]):
             pieces_step(hmm, seqs, alpha1, alpha2, inst, t)
         pieces_total(hmm, seqs, result, alpha1, alpha2, inst)
+
+
+@parpy.jit
+def strided_guarded_pick(a, b, out, N):
+    """512 iterations on 64 threads: thread g runs i = g, g + 64, ...; `a` has 48 elements, the test guards its index."""
+    parpy.label('i')
+    for i in range(N):
+        out[i] = (a[i % 64] if i % 64 < 48 else float32(-1.0)) + b[i // 64]

@@ -370,6 +370,34 @@ def test_scaled_reference_model_step_is_written_out_and_moves_whole_layer_rows()
     assert len(re.findall(r"const parpy_vec4<float> pk_\d+ = \*\(const parpy_vec4<float>\*\)&(parpy_at\()?hmm_pemit_", step1)) == 4
 
 
+def test_what_the_iterations_of_one_thread_share_is_evaluated_once_per_thread():
+    """The reference's kernel on a model whose state vector needs several workgroups, one thread per k-mer (4096
+    threads, 16 layers each): the loop variable is `g + k * 4096`, so the predecessors, their table rows, their
+    scores in the source vector (a local pointer that never names the array the loop stores to) and the emission
+    depend on g alone and are loaded in front of the counted loop; `state // 4096` is the counter itself."""
+    args = _reference_format_args(6, n=2, maxlen=6)
+    hmm = {k: v for k, v in args[0].items() if not k.startswith("p") and k != "log_emit_scale"}
+    a = np.zeros((2, hmm["num_states"]), dtype=np.float32)
+    call = [hmm, args[1], a, a.copy(), np.zeros(2, dtype=np.float32)]
+    o = opts_for({'inst': parpy.threads(2), 'state': parpy.threads(4096)})
+    s = compiles(parpy.print_compiled(W.forward_kernel, call, o))
+    step = [f for f in s.split("extern \"C\" __global__") if "alpha_src_" in f and "__builtin_amdgcn_logf" in f][0]
+    head, loop = step[:step.index("for (int state_")], step[step.index("for (int state_"):]
+    loop = loop[:loop.index("} else {")]
+    assert re.search(r"int state_\d+_g = \(\(int\)blockIdx.x \* 1024 \+ \(int\)threadIdx.x\);", head)
+    assert len(re.findall(r"float own_\d+ = alpha_src_\d+\[", head)) == 4 and len(re.findall(r"float t1\d_\d+ = ", head)) == 4
+    assert re.search(r"float own_\d+ = (parpy_at\()?hmm_output_prob_", head)
+    assert re.search(r"int state_\d+ = \(state_\d+_g \+ state_\d+_k \* 4096\);", loop)
+    assert len(re.findall(r"alpha_src_\d+\[", loop)) == 1          # what comes down from the layer above
+    assert " / " not in loop and " % " not in loop and re.search(r"hmm_trans2_\d+, \(unsigned\)\(state_\d+_k\)", loop)
+    s0 = compiles(parpy.print_compiled(W.forward_kernel, call, opts_for({'inst': parpy.threads(2), 'state': parpy.threads(4096)}, opt_share_iterations=False)))
+    assert "_g = " not in s0 and "float own_" not in s0
+    # an operand that a selection may skip stays inside the selection
+    x = np.zeros(48, dtype=np.float32)
+    s1 = compiles(parpy.print_compiled(K.strided_guarded_pick, [x, np.zeros(8, dtype=np.float32), np.zeros(512, dtype=np.float32), 512], opts_for({'i': parpy.threads(64)})))
+    assert re.search(r"\? a_\d+\[", s1) or re.search(r"\? parpy_at\(a_\d+", s1)
+
+
 def test_noalias_scope_wraps_the_step_body_when_aliases_never_coincide():
     hmm, seqs, args = _hmm_args(4)
     o = opts_for({'inst': parpy.threads(4), 'state': parpy.threads(256)}, opt_noalias_scopes=True)

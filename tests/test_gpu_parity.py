@@ -243,6 +243,19 @@ def test_reference_model_with_state_vectors_larger_than_lds(threads):
     assert np.all(np.isfinite(want)) and np.allclose(got, want, atol=1e-4, rtol=1e-5), np.abs(got - want).max()
 
 
+@pytest.mark.parametrize("threads", [4096, 16384])
+def test_reference_model_one_thread_per_kmer_shares_work_between_its_layers(threads):
+    """65536 states on 4096 threads per read (one per k-mer, 16 layers each) and on 16384 (four layers each): what
+    the layers of a k-mer have in common is evaluated once per thread; same operations on the same values, so the
+    results are bit-equal to those without the pass, and they match the oracle."""
+    hmm, seqs = _random_reference_model(6, n_reads=5, max_len=40, seed=23)
+    got = _run_reference_model(hmm, seqs, threads)
+    plain = _run_reference_model(hmm, seqs, threads, opt_share_iterations=False)
+    want = oracle.hmm_ref_forward(hmm, seqs, np.float32)
+    assert np.array_equal(got, plain)
+    assert np.all(np.isfinite(want)) and np.allclose(got, want, atol=1e-4, rtol=1e-5), np.abs(got - want).max()
+
+
 @pytest.mark.parametrize("k,threads", [(1, 64), (2, 100), (3, 192), (3, 640), (4, 1024), (4, 2048)])
 def test_reference_format_models_with_random_tables(k, threads):
     """Random tables in the reference model's layout, thread counts that do and do not divide the state count."""

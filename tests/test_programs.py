@@ -280,3 +280,18 @@ def test_groups_of_four_adjacent_elements(pack):
     w2 = w1 * np.float32(2)
     w3 = w2 - np.float32(3)
     assert np.array_equal(c.reshape(N, 4), np.stack([w3 * np.float32(0.5), w1, w2, w3], axis=1))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("share", [True, False], ids=["shared", "plain"])
+def test_strided_iterations_of_one_thread_with_a_guarded_index(share):
+    """512 iterations on 64 threads (thread g runs g, g + 64, ...): `a[i % 64]` is the same element in all of a
+    thread's iterations but only exists for i % 64 < 48, `b[i // 64]` is the iteration counter's element."""
+    import kernels as K
+    rng = np.random.default_rng(4)
+    a, b = rng.standard_normal(48).astype(np.float32), rng.standard_normal(8).astype(np.float32)
+    out = np.zeros(512, dtype=np.float32)
+    K.strided_guarded_pick(a, b, out, 512, opts=opts_for({'i': parpy.threads(64)}, opt_share_iterations=share))
+    i = np.arange(512)
+    want = np.where(i % 64 < 48, a[np.minimum(i % 64, 47)], np.float32(-1.0)) + b[i // 64]
+    assert np.array_equal(out, want.astype(np.float32))
