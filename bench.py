@@ -1,7 +1,7 @@
 """Benchmark of the compiled hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
-                    [--workload all|hmm7|hmm5|hmm5ref|rowsum|softmax|sddmm|copy] [--form scaled|grouped|reference]
+                    [--workload all|hmm7|hmm5|hmm5ref|hmm7ref|rowsum|softmax|sddmm|copy] [--form scaled|grouped|reference]
 
 A step is one pass of the compiled function over one batch of seeded synthetic
 input that is already resident in HBM.  The default run (`all`) times the
@@ -237,6 +237,57 @@ def bench_hmm_ref(args, torch, parpy, W, default_cfg=True):
     }
 
 
+def bench_hmm_ref7(args, torch, parpy, W, default_cfg=True):
+    """The reference's kernel (forward_kernel, test/test_forward.py:83-160) on a model of its 7-mer size: 16 layers x
+    16384 k-mers = 262144 states, a state vector of 1 MiB per read that cannot stay in LDS, so every step is one
+    launch over all reads with the state vectors in global memory (time loop on the host).  The reference ships no
+    7-mer tables; tables and reads are seeded random data in its format (100 reads of 500..1500 samples).  One
+    thread per k-mer: the 16 layers of a k-mer are the iterations of one thread."""
+    import numpy as np
+    import oracle
+    hmm, seqs = W.random_reference_model(7)
+    S, n = hmm["num_states"], seqs["num_instances"]
+    hd, sd = W.to_device(hmm), W.to_device(seqs)
+    a1 = torch.zeros((n, S), dtype=torch.float32, device="cuda")
+    a2 = torch.zeros_like(a1)
+    res = torch.zeros(n, dtype=torch.float32, device="cuda")
+    nthreads = args.state_threads if args.state_threads > 1024 else S // 16
+    opts = parpy.par({"inst": parpy.threads(n), "state": parpy.threads(nthreads)})
+    _apply_opt_flags(opts, args)
+    opts.use_cuda_graphs = bool(args.use_graphs)
+    opts.persistent_loops = bool(args.persistent)
+    fn = lambda: W.forward_kernel(hd, sd, a1, a2, res, opts=opts)
+    timed = lambda: parpy.time_call(W.forward_kernel, hd, sd, a1, a2, res, opts=opts)
+    steps = max(2, args.steps // 3)
+    wall, dev = _events_ms(fn, timed, steps, min(args.warmup, 2), torch)
+    got = res.cpu().numpy()
+    sub = np.argsort(seqs["lens"])[:4]
+    want = oracle.hmm_ref_forward(hmm, seqs, np.float32, subset=list(sub))
+    err = float(np.abs(got[sub] - want).max())
+    assert np.all(np.isfinite(got)) and np.allclose(got[sub], want, atol=1e-5, rtol=1e-5), err
+    steps_total = int((seqs["lens"] - 1).sum())
+    longest = int(seqs["lens"].max()) - 1
+    # per (read, step): alpha read + alpha write (4S each), one emission row of S/16 k-mers, the observation byte
+    alg_bytes = (8 * S + 4 * (S // 16) + 1) * steps_total
+    kernel_ms = float(np.median(dev))
+    roof = _hbm_roofline(alg_bytes, kernel_ms, "hmm7ref", default_cfg)
+    if roof["traffic"]:
+        roof["traffic"] *= longest   # the profile holds the mean over the step launches; a call makes one per step
+    roof["note"] = ("kernel_ms is the whole call: one launch per step over all reads that are still running "
+                    f"({longest} steps, {kernel_ms * 1e3 / longest:.1f} us per step)")
+    return {
+        "metric": "HMM-forward, model of the reference's 7-mer size (262144 states) ms/batch + achieved HBM GB/s (% of peak), 1xMI355X",
+        "value": wall, "unit": "ms/batch", "ms_per_step": wall, "higher_is_better": False, "dtype": "f32",
+        "config": {"workload": "hmm_forward_reference_format_7mer_random_tables", "form": "reference (forward_kernel)", "states": S,
+                   "reads": n, "min_len": int(seqs["lens"].min()), "max_len": int(seqs["lens"].max()), "total_steps": steps_total,
+                   "state_threads": nthreads, "steps_of_the_longest_read": longest, "graph_replay": bool(args.use_graphs),
+                   "checked": f"4 shortest reads against the fp32 oracle (atol = rtol = 1e-5), max abs error {err:.3g}"},
+        "roofline": roof,
+        "cpu_baseline": None,
+        "data": "seeded random tables in the reference's model format",
+    }
+
+
 def bench_rowsum(args, torch, parpy, W, default_cfg=True):
     import numpy as np
     N, M = 1024, 65536
@@ -408,7 +459,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="all", choices=["all", "hmm7", "hmm5", "hmm5ref", "rowsum", "softmax", "sddmm", "copy"])
+    ap.add_argument("--workload", default="all", choices=["all", "hmm7", "hmm5", "hmm5ref", "hmm7ref", "rowsum", "softmax", "sddmm", "copy"])
     ap.add_argument("--form", default="scaled", choices=["scaled", "grouped", "reference"],
                     help="which statement of the HMM step is the record's value (the others are timed beside it)")
     ap.add_argument("--single-form", action="store_true", help="time only the chosen form of the HMM step (profiling runs)")
@@ -440,6 +491,7 @@ def main():
         "hmm7": lambda: bench_hmm(7, args, torch, parpy, W, default_cfg),
         "hmm5": lambda: bench_hmm(5, args, torch, parpy, W, default_cfg),
         "hmm5ref": lambda: bench_hmm_ref(args, torch, parpy, W, default_cfg),
+        "hmm7ref": lambda: bench_hmm_ref7(args, torch, parpy, W, default_cfg),
         "rowsum": lambda: bench_rowsum(args, torch, parpy, W, default_cfg),
         "softmax": lambda: bench_softmax(args, torch, parpy, W, default_cfg),
         "sddmm": lambda: bench_sddmm(args, torch, parpy, W, default_cfg),
@@ -451,7 +503,7 @@ def main():
         r.update(common)
         r.setdefault("data", "synthetic")
         r["secondary"] = []
-        for w in ("hmm5", "hmm5ref", "rowsum", "softmax", "sddmm"):
+        for w in ("hmm5", "hmm5ref", "hmm7ref", "rowsum", "softmax", "sddmm"):
             s = runners[w]()
             s.setdefault("data", "synthetic")
             r["secondary"].append(s)

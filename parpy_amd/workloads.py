@@ -594,6 +594,27 @@ def load_reference_model(model_npz, signals_npz):
     return hmm, seqs
 
 
+def random_reference_model(k, n_reads=100, min_len=500, max_len=1500, seed=SEED, tail=0.05):
+    """Seeded random tables in the format of the reference's 16-layer model (`load_reference_model`) for sizes it
+    ships no tables for (its 7-mer model file is absent): Dirichlet rows for the successor, duration and emission
+    probabilities, uniform start over the first layer; reads of uniform random levels and lengths."""
+    rng = np.random.default_rng(seed)
+    nk = 4 ** k
+    hmm = {
+        "trans1": np.log(rng.dirichlet(np.ones(4), size=nk)).astype(np.float32),
+        "trans2": np.log(rng.dirichlet(np.ones(16))).astype(np.float32),
+        "output_prob": np.ascontiguousarray(np.log(rng.dirichlet(np.ones(101), size=nk)).T.astype(np.float32)),
+        "initial_prob": np.concatenate([np.full(nk, -np.log(float(nk))), np.full(15 * nk, -np.inf)]).astype(np.float32),
+        "gamma": np.float32(np.log(tail)),
+        "synthetic_248": np.float32(np.log1p(-tail)),
+        "num_states": 16 * nk,
+    }
+    lens = rng.integers(min_len, max_len + 1, size=n_reads).astype(np.int64)
+    data = rng.integers(0, 101, size=(n_reads, int(lens.max()))).astype(np.int8)
+    seqs = {"data": data, "lens": lens, "maxlen": int(lens.max()), "num_instances": n_reads}
+    return hmm, seqs
+
+
 def with_linear_tables(hmm):
     """The model with its transition tables also in linear space (`ptrans1`, `pstay`), as `forward_syn4` reads them."""
     out = dict(hmm)
