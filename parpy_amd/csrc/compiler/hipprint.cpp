@@ -678,8 +678,8 @@ struct DevicePrinter {
         gr.lo = 0;
         gr.hi = N - 1;
         ranges[Name{v + "_g", 0}] = gr;
-        narrow_vars.insert(Name{v + "_g", 0});
-        os << ind(n) << "int " << v << "_g = " << idx << ";\n";
+        if (narrow) narrow_vars.insert(Name{v + "_g", 0});
+        os << ind(n) << vty << " " << v << "_g = " << idx << ";\n";
         pstmts(s->els, n);
       }
       if (s->unroll) {

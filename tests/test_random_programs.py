@@ -183,3 +183,93 @@ def test_random_programs_on_device(case):
             parpy.jit(f)(*got, N, M, opts=opts_for(p))
             for g, w, label in zip(got, want, "xyz oO"):
                 assert np.allclose(g, w, rtol=1e-4, atol=1e-4, equal_nan=True), (src, N, M, sorted(p), label, np.abs(g - w).max())
+
+
+# ---------------------------------------------------------------- strided iterations with quotients and remainders
+def strided_program(rng, case, T):
+    """A parallel loop of 2T..8T iterations meant for T threads: thread g gets g, g + T, ...  Elements are picked by
+    quotients and remainders of the iteration number, some by divisors of T (the same element in all iterations of a
+    thread, or the counter's element) and some not; one term is a selection whose test guards an index."""
+    name = f"strided_{case}"
+    div = [1, 2, 4, T // 4, T // 2, T, 2 * T, 3, 5, 7]
+
+    def c():
+        return int(rng.choice(div))
+
+    def idx():
+        kind = int(rng.integers(0, 6))
+        if kind == 0:
+            return f"(i // {c()}) % {c()}"
+        if kind == 1:
+            return f"i % {c()}"
+        if kind == 2:
+            return f"(i % {c()}) // {int(rng.choice([1, 2, 3, 4]))}"
+        if kind == 3:
+            return f"((i // 4) % {max(T // 4, 1)}) + {int(rng.integers(0, 4))} * {max(T // 4, 1)}"
+        if kind == 4:
+            return f"(i // {int(rng.choice([T, 2 * T, T // 2]))}) * 3 + i % 3"
+        return f"(i + {int(rng.integers(1, 9))}) % {c()}"
+
+    def term():
+        kind = int(rng.integers(0, 5))
+        if kind == 0:
+            return f"a[{idx()}]"
+        if kind == 1:
+            return f"b[{idx()}] * a[{idx()}]"
+        if kind == 2:
+            return f"ops.float32(({idx()}) % 11)"
+        if kind == 3:
+            g = int(rng.choice([T // 2, T // 4 * 3]))
+            return f"(s[i % {T}] if i % {T} < {g} else b[{idx()}])"
+        return f"ops.max(a[{idx()}], b[i // {T}])"
+    body = " + ".join(term() for _ in range(int(rng.integers(2, 5))))
+    # (stored transposed -- thread g writes out[g * per + k] -- so that the loop keeps its strided form: a unit-stride
+    # store would have the iterations regrouped four to a thread)
+    src = (f"def {name}(a, b, s, out, N):\n    parpy.label('i')\n    for i in range(N):\n"
+           f"        out[(i % {T}) * (N // {T}) + i // {T}] = {body}\n")
+    return name, src
+
+
+STRIDED = list(range(24))
+
+
+def strided_inputs(rng, T, per):
+    N = T * per
+    # `s` is only as long as the widest guard allows (3 T / 4 elements): an unguarded read runs past it
+    return (rng.uniform(-1, 1, 16 * T + 64).astype(np.float32), rng.uniform(-1, 1, 16 * T + 64).astype(np.float32),
+            rng.uniform(-1, 1, T // 4 * 3).astype(np.float32), np.zeros(N, dtype=np.float32)), N
+
+
+@pytest.mark.parametrize("case", STRIDED[:8])
+def test_strided_programs_compile(case):
+    rng = np.random.default_rng(3000 + case)
+    T = int(rng.choice([64, 128, 256]))
+    name, src = strided_program(rng, case, T)
+    f = build(name, src)
+    arrays, N = strided_inputs(rng, T, 4)
+    for share in (True, False):
+        o = opts_for({'i': parpy.threads(T)})
+        o.opt_share_iterations = share
+        s = parpy.print_compiled(f, list(arrays) + [N], o)
+        hiprtc_compile(s[:s.index("// host side")], opts_for({}))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", STRIDED)
+def test_strided_programs_on_device(case):
+    rng = np.random.default_rng(3000 + case)
+    T = int(rng.choice([64, 128, 256]))
+    name, src = strided_program(rng, case, T)
+    f = build(name, src)
+    for per, tpb in [(2, None), (4, None), (8, 64), (3, None)]:
+        arrays, N = strided_inputs(rng, T, per)
+        want = [a.copy() for a in arrays]
+        f(*want, N)
+        for share in (True, False):
+            got = [a.copy() for a in arrays]
+            p = parpy.threads(T) if tpb is None else parpy.threads(T).tpb(tpb)
+            o = opts_for({'i': p})
+            o.opt_share_iterations = share
+            parpy.jit(f)(*got, N, opts=o)
+            # (products and sums may be contracted into fused multiply-adds on the device: not bit-equal)
+            assert np.allclose(got[-1], want[-1], rtol=1e-5, atol=1e-6), (src, T, per, tpb, share, np.abs(got[-1] - want[-1]).max())
