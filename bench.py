@@ -1,7 +1,7 @@
 """Benchmark of the compiled hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
-                    [--workload all|hmm7|hmm5|hmm5ref|hmm7ref|rowsum|softmax|sddmm|copy] [--form scaled|grouped|reference]
+                    [--workload all|hmm7|hmm5|hmm5ref|hmm7ref|rowsum|softmax|sddmm|copy|ldsrates] [--form scaled|grouped|reference]
 
 A step is one pass of the compiled function over one batch of seeded synthetic
 input that is already resident in HBM.  The default run (`all`) times the
@@ -50,6 +50,17 @@ HMM_VALU_MIX = {
     "scaled": {"full": 8.4, "trans": 0.0},
 }
 HMM_FORMS = {"scaled": "forward_scaled", "grouped": "forward_syn4", "reference": "forward_syn"}
+# LDS bytes per clock and compute unit measured with LDS-only microkernels on this part (1024 threads, 2.4 GHz):
+# 4-byte reads 102, 8- and 16-byte reads 193, 4-byte writes 61, 16-byte writes 75.  Per state and step the grouped
+# and scaled forms read one predecessor word (4-byte reads) and their own state (16-byte reads) and write their
+# state (16-byte writes); the reference form reads five words and writes one with 4-byte accesses.
+LDS_BYTES_PER_CLK = {"read32": 102.0, "read128": 193.0, "write32": 61.0, "write128": 75.0}
+LDS_CLK_GHZ = 2.4
+HMM_LDS_MIX = {
+    "reference": {"read32": 20, "write32": 4},
+    "grouped": {"read32": 4, "read128": 4, "write128": 4},
+    "scaled": {"read32": 4, "read128": 4, "write128": 4},
+}
 
 
 def _events_ms(fn, timed, steps, warmup, torch):
@@ -114,10 +125,16 @@ def bench_hmm(k, args, torch, parpy, W, default_cfg=True):
         mix = HMM_VALU_MIX[form]
         rows_per_simd = S / 256.0
         bound_ms = longest * rows_per_simd * (mix["full"] * VALU_NS["full"] + mix["trans"] * VALU_NS["trans"]) * 1e-6
+        clk_per_state = sum(b / LDS_BYTES_PER_CLK[kind] for kind, b in HMM_LDS_MIX[form].items())
+        lds_ms = longest * S * clk_per_state / (LDS_CLK_GHZ * 1e9) * 1e3
         forms[form] = {"wall": wall, "kernel_ms": kernel_ms, "ll": ll, "threads": threads,
                        "valu_bound": {"ms": bound_ms, "frac": bound_ms / kernel_ms,
                                       "model": f"{longest} steps of the longest read x {rows_per_simd:g} rows of 64 states per SIMD x "
-                                               f"({mix['full']} full-rate x {VALU_NS['full']} ns + {mix['trans']} exp/log x {VALU_NS['trans']} ns)"}}
+                                               f"({mix['full']} full-rate x {VALU_NS['full']} ns + {mix['trans']} exp/log x {VALU_NS['trans']} ns)"},
+                       "lds_bound": {"ms": lds_ms, "frac": lds_ms / kernel_ms,
+                                     "model": f"{longest} steps of the longest read x {S} states x "
+                                              + " + ".join(f"{b} B {kind} at {LDS_BYTES_PER_CLK[kind]:g} B/clk" for kind, b in HMM_LDS_MIX[form].items())
+                                              + f" on one compute unit at {LDS_CLK_GHZ} GHz (measured LDS rates)"}}
     # outside the timed region: the shortest reads at full length against the fp64 oracle (what the GPU tests do for all)
     sub = np.argsort(seqs["lens"])[:6]
     want = oracle.hmm_syn_forward(hmm, seqs, np.float64, subset=sub)
@@ -144,12 +161,16 @@ def bench_hmm(k, args, torch, parpy, W, default_cfg=True):
     resident = LDS_RESIDENT_NOTE if main["threads"] <= 1024 and 8 * S <= 156 * 1024 else None
     roof = _hbm_roofline(alg_bytes, main["kernel_ms"], f"hmm{k}{suffix[args.form]}", default_cfg, resident)
     roof["valu_bound"] = main["valu_bound"]
+    if resident:
+        roof["lds_bound"] = main["lds_bound"]
     other_forms = []
     for other in others:
         alt = forms[other]
         alt_roof = _hbm_roofline(alg_bytes, alt["kernel_ms"], f"hmm{k}{suffix[other]}", default_cfg,
                                  LDS_RESIDENT_NOTE if alt["threads"] <= 1024 and 8 * S <= 156 * 1024 else None)
         alt_roof["valu_bound"] = alt["valu_bound"]
+        if "note" in alt_roof:
+            alt_roof["lds_bound"] = alt["lds_bound"]
         other_forms.append({"form": f"{other} ({name[other]})", "ms_per_step": alt["wall"], "state_threads": alt["threads"],
                             "dtype": "f32 state vectors, " + ("f64 result" if other == "scaled" else "f32 result"),
                             "roofline": alt_roof, "checked_max_abs_error": checked[other]})
@@ -286,6 +307,116 @@ def bench_hmm_ref7(args, torch, parpy, W, default_cfg=True):
         "cpu_baseline": None,
         "data": "seeded random tables in the reference's model format",
     }
+
+
+LDS_RATE_KERNELS = r'''
+typedef float f4 __attribute__((ext_vector_type(4)));
+extern "C" __global__ void __launch_bounds__(1024) lds_read128(float* out, int iters) {
+  __shared__ f4 buf[4096];
+  for (int i = threadIdx.x; i < 4096; i += 1024) buf[i] = f4{(float)i, 1.0f, 2.0f, 3.0f};
+  __syncthreads();
+  f4 acc = {0, 0, 0, 0};
+  volatile __attribute__((address_space(3))) f4* vb = (__attribute__((address_space(3))) f4*)buf + threadIdx.x;
+  for (int it = 0; it < iters; ++it) {
+    f4 a = vb[0], b = vb[1024], c = vb[2048], d = vb[3072];
+    acc += (a + b) + (c + d);
+  }
+  out[blockIdx.x * 1024 + threadIdx.x] = acc.x + acc.y + acc.z + acc.w;
+}
+extern "C" __global__ void __launch_bounds__(1024) lds_read32(float* out, int iters) {
+  __shared__ float buf[16384];
+  for (int i = threadIdx.x; i < 16384; i += 1024) buf[i] = (float)i;
+  __syncthreads();
+  float acc = 0;
+  volatile __attribute__((address_space(3))) float* vb = (__attribute__((address_space(3))) float*)buf + threadIdx.x;
+  for (int it = 0; it < iters; ++it) {
+    float s = 0;
+    #pragma unroll
+    for (int k = 0; k < 16; ++k) s += vb[k * 1024];
+    acc += s;
+  }
+  out[blockIdx.x * 1024 + threadIdx.x] = acc;
+}
+extern "C" __global__ void __launch_bounds__(1024) lds_write128(float* out, int iters) {
+  __shared__ f4 buf[4096];
+  f4 v = {1.0f, 2.0f, 3.0f, (float)threadIdx.x};
+  volatile __attribute__((address_space(3))) f4* vb = (__attribute__((address_space(3))) f4*)buf + threadIdx.x;
+  for (int it = 0; it < iters; ++it) {
+    vb[0] = v; vb[1024] = v; vb[2048] = v; vb[3072] = v;
+    v.x += 1.0f;
+  }
+  __syncthreads();
+  out[blockIdx.x * 1024 + threadIdx.x] = buf[threadIdx.x].x;
+}
+
+typedef float f2 __attribute__((ext_vector_type(2)));
+extern "C" __global__ void __launch_bounds__(1024) lds_write32(float* out, int iters) {
+  __shared__ float buf[16384];
+  float v = (float)threadIdx.x;
+  volatile __attribute__((address_space(3))) float* vb = (__attribute__((address_space(3))) float*)buf + threadIdx.x;
+  for (int it = 0; it < iters; ++it) {
+    #pragma unroll
+    for (int k = 0; k < 16; ++k) vb[k * 1024] = v;
+    v += 1.0f;
+  }
+  __syncthreads();
+  out[blockIdx.x * 1024 + threadIdx.x] = buf[threadIdx.x];
+}
+extern "C" __global__ void __launch_bounds__(1024) lds_write64(float* out, int iters) {
+  __shared__ f2 buf[8192];
+  f2 v = {1.0f, (float)threadIdx.x};
+  volatile __attribute__((address_space(3))) f2* vb = (__attribute__((address_space(3))) f2*)buf + threadIdx.x;
+  for (int it = 0; it < iters; ++it) {
+    #pragma unroll
+    for (int k = 0; k < 8; ++k) vb[k * 1024] = v;
+    v.x += 1.0f;
+  }
+  __syncthreads();
+  out[blockIdx.x * 1024 + threadIdx.x] = buf[threadIdx.x].x;
+}
+extern "C" __global__ void __launch_bounds__(1024) lds_read64(float* out, int iters) {
+  __shared__ f2 buf[8192];
+  for (int i = threadIdx.x; i < 8192; i += 1024) buf[i] = f2{(float)i, 1.0f};
+  __syncthreads();
+  f2 acc = {0, 0};
+  volatile __attribute__((address_space(3))) f2* vb = (__attribute__((address_space(3))) f2*)buf + threadIdx.x;
+  for (int it = 0; it < iters; ++it) {
+    f2 s = {0, 0};
+    #pragma unroll
+    for (int k = 0; k < 8; ++k) s += vb[k * 1024];
+    acc += s;
+  }
+  out[blockIdx.x * 1024 + threadIdx.x] = acc.x + acc.y;
+}
+'''
+
+
+def bench_lds_rates(args, torch, parpy, W, default_cfg=True):
+    """LDS bytes per clock and compute unit for 4-, 8- and 16-byte reads and writes: hand-written microkernels (the
+    only ones in this file; everything else is compiled from ParPy user code) whose loops touch nothing but
+    registers and LDS, 1024 threads per workgroup, one workgroup per compute unit.  These are the rates behind
+    `lds_bound` of the HMM records."""
+    o = parpy.CompileOptions()
+    o.backend = parpy.CompileBackend.Hip
+    iters, blocks = 20000, 100
+    out = torch.zeros(blocks * 1024, dtype=torch.float32, device="cuda")
+    rates = {}
+    for name in ("lds_read32", "lds_read64", "lds_read128", "lds_write32", "lds_write64", "lds_write128"):
+        f = parpy.compile_string(name, LDS_RATE_KERNELS, o, grid=(blocks, 1, 1), block=(1024, 1, 1))
+        f(out, 10)
+        parpy.sync(o.backend)
+        ts = []
+        for _ in range(5):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            f(out, iters)
+            parpy.sync(o.backend)
+            ts.append(time.perf_counter() - t0)
+        per_cu = 1024 * 64 * iters / sorted(ts)[2]        # every thread moves 64 bytes per iteration
+        rates[name] = {"GB/s per CU": per_cu / 1e9, "B/clk at 2.4 GHz": per_cu / (LDS_CLK_GHZ * 1e9)}
+    return {"metric": "LDS bytes per clock and compute unit, 1xMI355X", "value": rates["lds_read128"]["B/clk at 2.4 GHz"], "unit": "B/clk/CU",
+            "ms_per_step": None, "higher_is_better": True, "dtype": "f32", "config": {"workload": "lds_rates", "rates": rates},
+            "roofline": None, "cpu_baseline": None}
 
 
 def bench_rowsum(args, torch, parpy, W, default_cfg=True):
@@ -459,7 +590,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="all", choices=["all", "hmm7", "hmm5", "hmm5ref", "hmm7ref", "rowsum", "softmax", "sddmm", "copy"])
+    ap.add_argument("--workload", default="all", choices=["all", "hmm7", "hmm5", "hmm5ref", "hmm7ref", "rowsum", "softmax", "sddmm", "copy", "ldsrates"])
     ap.add_argument("--form", default="scaled", choices=["scaled", "grouped", "reference"],
                     help="which statement of the HMM step is the record's value (the others are timed beside it)")
     ap.add_argument("--single-form", action="store_true", help="time only the chosen form of the HMM step (profiling runs)")
@@ -496,6 +627,7 @@ def main():
         "softmax": lambda: bench_softmax(args, torch, parpy, W, default_cfg),
         "sddmm": lambda: bench_sddmm(args, torch, parpy, W, default_cfg),
         "copy": lambda: bench_copy(args, torch, parpy, W, default_cfg),
+        "ldsrates": lambda: bench_lds_rates(args, torch, parpy, W, default_cfg),
     }
     common = {"n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "scaling": "weak", "vs_baseline": None}
     if args.workload == "all":
