@@ -1052,6 +1052,18 @@ def test_persistent_step_loop_on_the_synthetic_model_and_fallback_when_the_grid_
     assert np.allclose(got, want, atol=1e-5, rtol=1e-5), np.abs(got - want).max()
 
 
+def test_persistent_step_loop_with_values_shared_between_a_threads_iterations():
+    """One thread per k-mer of a 65536-state model (16 layers = 16 iterations per thread, 16 workgroups per read)
+    with the time loop inside one kernel: what the iterations share is loaded at device scope in front of the
+    counted loop; results equal those of the loop of launches bit for bit."""
+    hmm, seqs = _random_reference_model(6, n_reads=3, max_len=25, seed=31)
+    plain = _run_reference_model(hmm, seqs, 4096)
+    got = _run_reference_model(hmm, seqs, 4096, persistent_loops=True)
+    want = oracle.hmm_ref_forward(hmm, seqs, np.float32)
+    assert np.array_equal(got, plain)
+    assert np.allclose(got, want, atol=1e-4, rtol=1e-5), np.abs(got - want).max()
+
+
 def test_persistent_step_loop_reports_a_barrier_that_times_out(monkeypatch):
     """With a poll limit of zero the first workgroup that has to wait gives up: every workgroup leaves the kernel
     (it ends normally) and the next synchronisation raises."""
