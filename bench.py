@@ -572,10 +572,10 @@ def _profiled_field(name, field):
 
 
 def _profiled_traffic(name):
-    """(HBM bytes per launch, where the figure comes from): FETCH_SIZE + WRITE_SIZE of the committed counter run of
-    the same command, not measured in this run."""
+    """(HBM bytes per launch, where the figure comes from): FETCH_SIZE + WRITE_SIZE of the committed counter runs of
+    the same kernel (the file gives their commands), not measured in this run."""
     v = _profiled_field(name, "traffic_bytes_per_launch")
-    return (v, f"profiles/{name}_kernel.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of an earlier run of this command)") if v else (None, None)
+    return (v, f"profiles/{name}_kernel.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of the same kernel, commands in that file)") if v else (None, None)
 
 
 def _apply_opt_flags(opts, args):
