@@ -553,3 +553,58 @@ def test_selects_on_the_iteration_alone_keep_their_values(threads):
         got_x, got_y = x0.copy(), np.zeros_like(x0)
         parpy.jit(relax)(got_x, got_y, N, M, T, opts=opts_for({'N': parpy.threads(N), 'M': parpy.threads(threads)}, **flags))
         assert np.allclose(got_x, want_x, rtol=1e-5, atol=1e-6) and np.allclose(got_y, want_y, rtol=1e-5, atol=1e-6), flags
+
+
+def test_rejections_the_reference_tests_for_contexts_dictionaries_returns_and_calls():
+    """test/test_unsupported.py:33-67,82-95 and test/test_call.py:97-137,207-223 of the reference: same exception
+    type and the same words in the message."""
+    import parpy_amd.types as types
+
+    with pytest.raises(RuntimeError, match=r"lines \d+-\d+"):
+        @parpy.jit
+        def with_context():
+            with 5:
+                pass
+
+    @parpy.jit
+    def dict_arg(a):
+        with parpy.gpu:
+            a["x"] = a["y"]
+    with pytest.raises(RuntimeError, match="non-string key"):
+        parpy.print_compiled(dict_arg, [{'x': 2, 'y': 4, 3: 5}], opts_for({}))
+
+    @parpy.jit
+    def f_return(x):
+        with parpy.gpu:
+            y = parpy.operators.sum(x[:])
+            return y
+    with pytest.raises(RuntimeError, match="The called function f_return cannot return a value"):
+        parpy.print_compiled(f_return, [np.zeros(10)], opts_for({}))
+
+    def non_decorated_add(x, y, M):
+        for i in range(M):
+            y[i] += x[i]
+    with pytest.raises(RuntimeError, match="unknown function non_decorated_add"):
+        @parpy.jit
+        def add_2d(x, y, N, M):
+            parpy.label('N')
+            for i in range(N):
+                non_decorated_add(x[i], y[i], M)
+
+    @parpy.external("_zero", parpy.CompileBackend.Cuda, parpy.Target.Device)
+    def zero() -> types.I32:
+        return 0
+
+    @parpy.jit
+    def uses_zero(x):
+        with parpy.gpu:
+            x[:] = zero()
+    with pytest.raises(RuntimeError, match="Call to unknown function zero"):
+        parpy.print_compiled(uses_zero, [np.zeros(10, dtype=np.int32)], opts_for({}))
+
+    @parpy.jit
+    def needs_opts(x):
+        with parpy.gpu:
+            x[0] = 1.0
+    with pytest.raises(RuntimeError, match="opts"):
+        needs_opts(np.zeros(4, dtype=np.float32))
