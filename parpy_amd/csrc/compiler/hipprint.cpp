@@ -357,6 +357,7 @@ struct DevicePrinter {
   // accesses that must be coherent across the device: global elements of arrays that a kernel with
   // device-wide barriers may write (everything that is not a read-only parameter)
   bool as_lvalue = false;
+  bool wide_division = false;   // set while printing an expression that contains a 64-bit quotient or remainder
   bool exchanged(const E& e) const {
     if (!kernel || !kernel->no_restrict || e->k != Expr::Index) return false;
     const E& base = e->args[0];
@@ -462,6 +463,22 @@ struct DevicePrinter {
             if (sz == ElemSize::F16) return std::string("((_Float16)f") + base + "f((float)" + paren(a) + ", (float)" + paren(b) + "))";
             return std::string("parpy_") + base + "<" + elem_ctype(sz) + ">(" + a + ", " + b + ")";
           }
+          case BinOp::FloorDiv: case BinOp::Div: case BinOp::Rem: {
+            // A quotient or remainder of 64-bit integers whose operands provably fit 31 bits is computed in 32
+            // bits (one multiply-high for a constant divisor instead of a 64-bit sequence).  The wide form is also
+            // kept out of 32-bit offsets (see `parpy_at`): a 64-bit division by a constant whose result was only
+            // used truncated to 32 bits has produced wrong element offsets on gfx950 (the same source with the
+            // 32-bit division is correct), so such an index stays a plain 64-bit one.
+            bool wide = e->ty.is_scalar() && (e->ty.sz == ElemSize::I64 || e->ty.sz == ElemSize::U64) && e->args[0]->ty.is_scalar() &&
+                        is_int(e->args[0]->ty.sz) && e->args[1]->ty.is_scalar() && is_int(e->args[1]->ty.sz);
+            if (wide) {
+              Interval ra = expr_range(e->args[0], ranges), rb = expr_range(e->args[1], ranges);
+              if (ra.known && rb.known && ra.lo >= 0 && ra.hi <= INT32_MAX && rb.lo > 0 && rb.hi <= INT32_MAX)
+                return "((" + std::string(elem_ctype(e->ty.sz)) + ")((int)" + paren(a) + " " + cop(e->bop) + " (int)" + paren(b) + "))";
+              wide_division = true;
+            }
+            return "(" + a + " " + cop(e->bop) + " " + b + ")";
+          }
           case BinOp::Atan2: return std::string(sz == ElemSize::F64 ? "atan2" : "atan2f") + "(" + a + ", " + b + ")";
           case BinOp::Pow: return std::string(sz == ElemSize::F64 ? "pow" : "__powf") + "(" + a + ", " + b + ")";
           default: return "(" + a + " " + cop(e->bop) + " " + b + ")";
@@ -518,8 +535,13 @@ struct DevicePrinter {
           // 10^5 floats: 0.7 ms against 1.1 ms).
           Interval r = expr_range(e->args[1], ranges);
           int64_t eb = elem_bytes(e->ty.sz);
-          if (r.known && r.lo >= 0 && r.hi * eb + eb <= (int64_t)UINT32_MAX)
-            out = "parpy_at(" + pexpr(e->args[0]) + ", (unsigned)(" + pexpr(e->args[1]) + "))";
+          if (r.known && r.lo >= 0 && r.hi * eb + eb <= (int64_t)UINT32_MAX) {
+            bool outer = wide_division;
+            wide_division = false;
+            std::string idx = pexpr(e->args[1]);
+            if (!wide_division) out = "parpy_at(" + pexpr(e->args[0]) + ", (unsigned)(" + idx + "))";
+            wide_division = wide_division || outer;
+          }
         }
         for (auto& n : assumed) ranges.erase(n);
         for (auto& kv : narrowed) ranges[kv.first] = kv.second;

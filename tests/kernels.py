@@ -247,3 +247,11 @@ def strided_guarded_pick(a, b, out, N):
     parpy.label('i')
     for i in range(N):
         out[i] = (a[i % 64] if i % 64 < 48 else float32(-1.0)) + b[i // 64]
+
+
+@parpy.jit
+def pick_by_quotients(a, idx, out, N):
+    """`i // 3` of a loop counter fits 31 bits; `idx[i] // 3` of a loaded 64-bit value does not provably."""
+    parpy.label('i')
+    for i in range(N):
+        out[i] = a[(i // 3) % 8] + a[(idx[i] // 3) % 8]

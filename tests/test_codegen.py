@@ -398,6 +398,17 @@ def test_what_the_iterations_of_one_thread_share_is_evaluated_once_per_thread():
     assert re.search(r"\? a_\d+\[", s1) or re.search(r"\? parpy_at\(a_\d+", s1)
 
 
+def test_quotients_are_taken_in_32_bits_where_they_fit_and_never_cut_down_to_an_offset_otherwise():
+    a, idx, out = np.zeros(8, dtype=np.float32), np.zeros(256, dtype=np.int64), np.zeros(256, dtype=np.float32)
+    s = compiles(parpy.print_compiled(K.pick_by_quotients, [a, idx, out, 256],
+                                      opts_for({'i': parpy.threads(64)}, opt_narrow_index=False, opt_vectorize=False)))
+    k = s[s.index('extern "C" __global__'):s.index("// host side")]
+    # the counter is a 64-bit variable here, but its quotient by 3 and the remainder by 8 fit: computed as int
+    assert re.search(r"\(int\)\(i_\d+\) / \(int\)", k) and re.search(r"parpy_at\(a_\d+, \(unsigned\)\(\(\(int64_t\)\(\(int\)", k)
+    # the loaded value has no such bound: 64-bit division, and the element is addressed with the plain 64-bit index
+    assert re.search(r"a_\d+\[\(\(parpy_at\(idx_\d+, \(unsigned\)\(i_\d+\)\) / \(\(int64_t\)3LL\)\) % \(\(int64_t\)8LL\)\)\]", k)
+
+
 def test_noalias_scope_wraps_the_step_body_when_aliases_never_coincide():
     hmm, seqs, args = _hmm_args(4)
     o = opts_for({'inst': parpy.threads(4), 'state': parpy.threads(256)}, opt_noalias_scopes=True)

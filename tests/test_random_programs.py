@@ -265,11 +265,14 @@ def test_strided_programs_on_device(case):
         arrays, N = strided_inputs(rng, T, per)
         want = [a.copy() for a in arrays]
         f(*want, N)
-        for share in (True, False):
+        # (with 64-bit index arithmetic as well: quotients and remainders of sums that provably fit 31 bits are
+        # computed in 32 bits, and no 64-bit quotient is ever cut down to a 32-bit element offset)
+        for share, narrow in ((True, True), (False, True), (True, False)):
             got = [a.copy() for a in arrays]
             p = parpy.threads(T) if tpb is None else parpy.threads(T).tpb(tpb)
             o = opts_for({'i': p})
             o.opt_share_iterations = share
+            o.opt_narrow_index = narrow
             parpy.jit(f)(*got, N, opts=o)
             # (products and sums may be contracted into fused multiply-adds on the device: not bit-equal)
-            assert np.allclose(got[-1], want[-1], rtol=1e-5, atol=1e-6), (src, T, per, tpb, share, np.abs(got[-1] - want[-1]).max())
+            assert np.allclose(got[-1], want[-1], rtol=1e-5, atol=1e-6), (src, T, per, tpb, share, narrow, np.abs(got[-1] - want[-1]).max())
