@@ -1,7 +1,7 @@
 """Benchmark of the compiled hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
-                    [--workload all|hmm7|hmm5|hmm5ref|hmm7ref|rowsum|softmax|sddmm|copy|ldsrates] [--form scaled|grouped|reference]
+                    [--workload all|hmm7|hmm5|hmm5ref|hmm7ref|rowsum|softmax|sddmm|copy|ldsrates|valurates] [--form scaled|grouped|reference]
 
 A step is one pass of the compiled function over one batch of seeded synthetic
 input that is already resident in HBM.  The default run (`all`) times the
@@ -41,9 +41,9 @@ OPT_FLAGS = ("opt_vectorize", "opt_lds_rows", "opt_reg_cache", "opt_hoist_invari
 
 # Vector-ALU instructions per state and step in the time loop of the generated HMM kernels (counted in the ISA of
 # the kernels as compiled for these shapes: full-rate instructions, and v_exp_f32 / v_log_f32), and the issue times
-# of the two classes measured with register-only microkernels on this part (4 waves per SIMD).  One workgroup of 16
+# of the two classes measured with register-only microkernels on this part (4 waves per SIMD; `--workload valurates`).  One workgroup of 16
 # waves per read puts S / 256 rows of 64 states on each SIMD.
-VALU_NS = {"full": 1.17, "trans": 3.76}
+VALU_NS = {"full": 1.02, "trans": 3.63}   # with 100 compute units busy, as in the HMM launches (1.15 / 3.77 with all 256)
 HMM_VALU_MIX = {
     "reference": {"full": 24.0, "trans": 6.0},
     "grouped": {"full": 14.2, "trans": 3.0},
@@ -421,6 +421,54 @@ def bench_lds_rates(args, torch, parpy, W, default_cfg=True):
             "roofline": None, "cpu_baseline": None}
 
 
+def _valu_rate_kernel(name, adds, exps):
+    """A loop whose body is `adds` independent v_add_f32 (eight accumulators) and `exps` independent v_exp_f32, registers only."""
+    lines = [f"v_add_f32 v{16 + i % 8}, v{16 + i % 8}, v{41 + i % 8}" for i in range(adds)]
+    lines += [f"v_exp_f32 v{24 + i % 8}, v{24 + i % 8}" for i in range(exps)]
+    body = "\\n".join(lines)
+    init = "\\n".join([f"v_mov_b32 v{r}, 0x3f000000" for r in range(40, 52)] + [f"v_mov_b32 v{r}, 0" for r in range(16, 32)])
+    clob = ", ".join(f'"v{r}"' for r in range(16, 32))
+    clob_all = ", ".join(f'"v{r}"' for r in list(range(16, 32)) + list(range(40, 52)))
+    return f'''
+extern "C" __global__ void __launch_bounds__(1024) {name}(float* out, int iters) {{
+  asm volatile("{init}" ::: {clob_all});
+  for (int i = 0; i < iters; ++i) {{
+    asm volatile("{body}" ::: {clob});
+  }}
+  float r, r2;
+  asm volatile("v_mov_b32 %0, v16\\nv_mov_b32 %1, v24" : "=v"(r), "=v"(r2));
+  out[blockIdx.x * 1024 + threadIdx.x] = r + r2;
+}}'''
+
+
+def bench_valu_rates(args, torch, parpy, W, default_cfg=True):
+    """Issue time of a full-rate vector instruction and of v_exp_f32 per wave with four waves on a SIMD (a
+    1024-thread workgroup on its compute unit): register-only microkernels.  These are `VALU_NS`, the times behind
+    `valu_bound` of the HMM records."""
+    o = parpy.CompileOptions()
+    o.backend = parpy.CompileBackend.Hip
+    iters, blocks = 20000, 100
+    out = torch.zeros(blocks * 1024, dtype=torch.float32, device="cuda")
+    res = {}
+    for name, adds, exps in (("valu_add32", 32, 0), ("valu_exp8", 0, 8)):
+        f = parpy.compile_string(name, _valu_rate_kernel(name, adds, exps), o, grid=(blocks, 1, 1), block=(1024, 1, 1))
+        f(out, 10)
+        parpy.sync(o.backend)
+        ts = []
+        for _ in range(5):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            f(out, iters)
+            parpy.sync(o.backend)
+            ts.append(time.perf_counter() - t0)
+        # four waves per SIMD take turns: the time of one instruction of one wave is the loop time over 4 x count
+        res[name] = sorted(ts)[2] * 1e9 / (iters * 4 * (adds + exps))
+    return {"metric": "vector-ALU issue time per wave instruction with 4 waves per SIMD, 1xMI355X", "value": res["valu_add32"], "unit": "ns",
+            "ms_per_step": None, "higher_is_better": False, "dtype": "f32",
+            "config": {"workload": "valu_rates", "v_add_f32_ns": res["valu_add32"], "v_exp_f32_ns": res["valu_exp8"]},
+            "roofline": None, "cpu_baseline": None}
+
+
 def bench_rowsum(args, torch, parpy, W, default_cfg=True):
     import numpy as np
     N, M = 1024, 65536
@@ -592,7 +640,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="all", choices=["all", "hmm7", "hmm5", "hmm5ref", "hmm7ref", "rowsum", "softmax", "sddmm", "copy", "ldsrates"])
+    ap.add_argument("--workload", default="all", choices=["all", "hmm7", "hmm5", "hmm5ref", "hmm7ref", "rowsum", "softmax", "sddmm", "copy", "ldsrates", "valurates"])
     ap.add_argument("--form", default="scaled", choices=["scaled", "grouped", "reference"],
                     help="which statement of the HMM step is the record's value (the others are timed beside it)")
     ap.add_argument("--single-form", action="store_true", help="time only the chosen form of the HMM step (profiling runs)")
@@ -630,6 +678,7 @@ def main():
         "sddmm": lambda: bench_sddmm(args, torch, parpy, W, default_cfg),
         "copy": lambda: bench_copy(args, torch, parpy, W, default_cfg),
         "ldsrates": lambda: bench_lds_rates(args, torch, parpy, W, default_cfg),
+        "valurates": lambda: bench_valu_rates(args, torch, parpy, W, default_cfg),
     }
     common = {"n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "scaling": "weak", "vs_baseline": None}
     if args.workload == "all":
