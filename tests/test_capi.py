@@ -70,3 +70,23 @@ def test_a_library_older_than_its_sources_is_loaded_with_a_warning_and_rebuilt_o
     monkeypatch.setenv("PARPY_AMD_REBUILD", "1")
     runtime.load_hip_runtime_lib()
     assert built == [False]
+
+
+def test_running_without_a_device_fails_loudly():
+    """No CPU path stands in for the HIP backend: with no ROCm device a call raises (the reference's messages,
+    python/parpy/backend.py), it does not fall back to anything."""
+    import numpy as np
+    import parpy_amd as parpy
+    if parpy.backend.is_enabled(parpy.CompileBackend.Hip):
+        pytest.skip("a ROCm device is visible")
+
+    @parpy.jit
+    def set_first(x):
+        with parpy.gpu:
+            x[0] = 1.0
+    o = parpy.par({})
+    o.backend = parpy.CompileBackend.Hip
+    with pytest.raises(RuntimeError, match="Specified backend CompileBackend.Hip is not available"):
+        set_first(np.zeros(4, dtype=np.float32), opts=o)
+    with pytest.raises(RuntimeError, match="Found no enabled GPU backends"):
+        set_first(np.zeros(4, dtype=np.float32), opts=parpy.par({}))
