@@ -550,6 +550,7 @@ def bench_sddmm(args, torch, parpy, W, default_cfg=True):
     zero = torch.tensor(0.0, dtype=torch.float32)
     opts = parpy.par({"nnz": parpy.threads(nnz).tpb(args.tpb)})
     _apply_opt_flags(opts, args)
+    opts.use_cuda_graphs = bool(args.use_graphs)
     fn = lambda: W.sddmm_coo(Ad, Bd, C, D, one, zero, opts=opts)
     timed = lambda: parpy.time_call(W.sddmm_coo, Ad, Bd, C, D, one, zero, opts=opts)
     wall, dev = _events_ms(fn, timed, args.steps, args.warmup, torch)
