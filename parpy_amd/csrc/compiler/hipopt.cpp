@@ -1277,6 +1277,12 @@ struct Pass {
     // working set fit without spilling (measured on the HMM kernels; 96 spills a few)
     if (threads <= 512) return threads <= 256 ? 192 : 128;
     // a per-element step body without exponentials or logarithms keeps few values alive besides the cached ones
+    return step_has_transcendentals() ? 88 : 104;
+  }
+
+  // whether the per-element body of a step loop (a thread-mapped loop inside a sequential loop) takes exponentials
+  // or logarithms: such a step is bound by the vector ALU, one without them by what it moves
+  bool step_has_transcendentals() const {
     bool transcendental = false;
     std::function<void(const Stmts&, bool, bool)> walk = [&](const Stmts& ss, bool in_seq, bool in_threads) {
       for (auto& st : ss) {
@@ -1296,7 +1302,7 @@ struct Pass {
       }
     };
     walk(k.body, false, false);
-    return transcendental ? 88 : 104;
+    return transcendental;
   }
 
   // hoist out of the sequential loop `seq` (a statement of `parent`)
@@ -2956,6 +2962,7 @@ void hip_optimize(Program& p, const Options& opts, NameGen& gen) {
     if (opts.opt_drop_barriers) pass.drop_barriers();
     k.distinct_pointers.clear();
     k.body = pass.noalias_scopes(k.body, opts.opt_noalias_scopes);
+    k.fence_lds_iterations = opts.opt_fence_iterations && !pass.step_has_transcendentals();
     pass.mark_read_only();
     k.aligned_params = opts.assume_aligned;
   }

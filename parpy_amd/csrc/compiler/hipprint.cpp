@@ -613,6 +613,21 @@ struct DevicePrinter {
     return r;
   }
 
+  static bool reads_and_writes_lds(const Stmts& body) {
+    bool rd = false, wr = false;
+    visit_stmts(body, [&](const S& c) {
+      if (c->k == Stmt::Assign && c->dst->k == Expr::Index && c->dst->args[0]->ty.mem == Mem::LDS) wr = true;
+      auto scan = [&](const E& root, bool skip_root) {
+        visit_exprs(root, [&](const E& x) {
+          if (x->k == Expr::Index && x->args[0]->ty.mem == Mem::LDS && !(skip_root && x.get() == root.get())) rd = true;
+        });
+      };
+      if (c->expr) scan(c->expr, false);
+      if (c->dst) scan(c->dst, c->k == Stmt::Assign);
+    });
+    return rd && wr;
+  }
+
   void pfor(const S& s, int n) {
     Interval lo = expr_range(s->lo, ranges), hi = expr_range(s->hi, ranges);
     bool is64 = s->lo->ty.is_scalar() && s->lo->ty.sz == ElemSize::I64;
@@ -723,6 +738,15 @@ struct DevicePrinter {
         os << ind(n + 2) << "}\n";
       } else {
         pstmts(s->body, n + 2);
+      }
+      if (kernel->fence_lds_iterations && s->unroll && per > 1 && reads_and_writes_lds(s->body)) {
+        // Left to itself the device compiler issues the LDS loads of all unrolled iterations first.  Every wave of
+        // the workgroup then queues at the LDS at the same moment (they have just left the same barrier) with the
+        // vector ALU idle, and computes afterwards with the LDS idle.  With the iterations kept apart the waves
+        // drift out of step and one wave's arithmetic covers another's LDS traffic (scaled 7-mer HMM step: 19.0 ->
+        // 17.8 ms per batch).  Only for steps without exponentials or logarithms: those are bound by the vector
+        // ALU and lose a little (reference form 56.8 -> 58.2 ms), the grouped form neither gains nor loses.
+        os << ind(n + 2) << "__builtin_amdgcn_sched_barrier(0);\n";
       }
       os << ind(n) << "}\n";
       if (shared_first) {
@@ -1074,6 +1098,7 @@ struct DevicePrinter {
         if (packs[p].owner == &ss && packs[p].is_store && packs[p].last == i) {
           if (packs[p].streamed) os << ind(n) << "__builtin_nontemporal_store(" << packs[p].var << ", " << packs[p].addr << ");\n";
           else os << ind(n) << "*" << packs[p].addr << " = " << packs[p].var << ";\n";
+
         }
     }
   }

@@ -95,6 +95,7 @@ Options parse_options(const std::string& sexpr) {
     else if (h == "opt_guard_bounds") o.opt_guard_bounds = flag();
     else if (h == "opt_pack_accesses") o.opt_pack_accesses = flag();
     else if (h == "opt_share_iterations") o.opt_share_iterations = flag();
+    else if (h == "opt_fence_iterations") o.opt_fence_iterations = flag();
     else if (h == "opt_prefetch_steps") o.opt_prefetch_steps = flag();
     else if (h == "reg_budget") o.reg_budget = f->at(1)->as_int();
     else if (h == "assume_aligned") o.assume_aligned = flag();

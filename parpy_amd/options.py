@@ -259,6 +259,7 @@ class CompileOptions:
         'opt_guard_bounds': None,
         'opt_pack_accesses': None,
         'opt_share_iterations': None,
+        'opt_fence_iterations': None,
         'opt_prefetch_steps': None,
         'reg_budget': None,   # registers per thread the caching passes may claim (None: by block size)
         'assume_aligned': None,   # set by the driver: False when an array argument is not 16-byte aligned

@@ -409,6 +409,28 @@ def test_quotients_are_taken_in_32_bits_where_they_fit_and_never_cut_down_to_an_
     assert re.search(r"a_\d+\[\(\(parpy_at\(idx_\d+, \(unsigned\)\(i_\d+\)\) / \(\(int64_t\)3LL\)\) % \(\(int64_t\)8LL\)\)\]", k)
 
 
+def test_unrolled_lds_iterations_of_a_step_without_transcendentals_are_kept_apart():
+    """The scaled 7-mer step gives every thread four groups (load from LDS, multiply-add, store to LDS): a
+    scheduling fence ends each unrolled iteration.  Steps with exponentials and logarithms (vector-ALU bound) and
+    loops of one iteration per thread do not get one."""
+    hmm, seqs = W.synthetic_hmm(7, n_inst=2, min_len=10, max_len=20)
+    S = hmm["num_states"]
+    b = np.zeros((2, S), dtype=np.float32)
+    o = opts_for({'inst': parpy.threads(2), 'state': parpy.threads(1024)})
+    s = compiles(parpy.print_compiled(W.forward_scaled, [W.with_scaled_tables(hmm), seqs, np.zeros(2), b, b.copy()], o))
+    step = s[s.index("for (int t_"):]
+    assert len(re.findall(r"= pk_\d+;\n\s+__builtin_amdgcn_sched_barrier\(0\);\n\s+\}", step)) == 1
+    off = compiles(parpy.print_compiled(W.forward_scaled, [W.with_scaled_tables(hmm), seqs, np.zeros(2), b, b.copy()],
+                                        opts_for({'inst': parpy.threads(2), 'state': parpy.threads(1024)}, opt_fence_iterations=False)))
+    assert "sched_barrier" not in off
+    for fn, res in ((W.forward_syn4, np.zeros(2, dtype=np.float32)), (W.forward_syn, np.zeros(2, dtype=np.float32))):
+        assert "sched_barrier" not in compiles(parpy.print_compiled(fn, [W.with_scaled_tables(hmm), seqs, res, b, b.copy()], o))
+    hmm5, seqs5 = W.synthetic_hmm(5, n_inst=2, min_len=10, max_len=20)
+    b5 = np.zeros((2, 1024), dtype=np.float32)
+    assert "sched_barrier" not in compiles(parpy.print_compiled(W.forward_scaled, [W.with_scaled_tables(hmm5), seqs5, np.zeros(2), b5, b5.copy()],
+                                                                 opts_for({'inst': parpy.threads(2), 'state': parpy.threads(256)})))
+
+
 def test_noalias_scope_wraps_the_step_body_when_aliases_never_coincide():
     hmm, seqs, args = _hmm_args(4)
     o = opts_for({'inst': parpy.threads(4), 'state': parpy.threads(256)}, opt_noalias_scopes=True)
