@@ -8,7 +8,7 @@ HIP backend -- nothing here calls a hand-written kernel.
 import numpy as np
 
 import parpy_amd as parpy
-from parpy_amd.operators import exp, float32, float64, inf, int32, log, max, min, sum
+from parpy_amd.operators import exp, float32, float64, inf, int32, int64, log, max, min, sum
 
 
 # ---------------------------------------------------------------- reductions / softmax
@@ -374,26 +374,38 @@ def forward_scaled_top(hmm, seqs, beta1, beta2, inst, t):
 
 
 @parpy.jit
+def scaled_doublings(top):
+    """How many times the state vector whose largest element is `top` can be doubled without passing one
+    (0 .. 62; nothing has to be exact here, any power of two near 1 / top serves as the divisor)."""
+    return int64(min(max(-log(top) * float32(1.4426950408889634), float32(0.0)), float32(62.0)))
+
+
+@parpy.jit
 def forward_scaled(hmm, seqs, result, beta1, beta2):
     """The forward pass of the synthetic model in linear space with rescaling (the classical alternative to
-    log space): beta[s] holds the probability alpha[s] times a running scale whose logarithm is kept in
-    float64.  Tables are probabilities: `ptrans1`, `pstay`, `pinit`, and `pemit` = emission probabilities
-    times the constant exp(`log_emit_scale`) that makes the largest of them one.  A step is one multiplication
-    and four multiply-adds per state for the sum over its predecessors and itself and two multiplications (by the
-    divisor `r` and by the emission), no exponential and no logarithm.  Every eighth step the largest element of
-    the new state vector is looked up; the vector itself is left alone and the next step divides what it
-    produces by that element (the step is linear, so this is the same as dividing its input, without a second
-    pass over the vector).  The divisors are collected as a float64 product whose logarithm is taken every 64
-    steps.  The result is float64:
-    log-likelihood = log(sum of the final vector) + sum of log(divisors) - len * log_emit_scale."""
+    log space): beta[s] holds the probability alpha[s] times a running scale.  Tables are probabilities:
+    `ptrans1`, `pstay`, `pinit`, and `pemit` = emission probabilities times the constant exp(`log_emit_scale`)
+    that makes the largest of them one.  A step is one multiplication and four multiply-adds per state for the
+    sum over its predecessors and itself and two multiplications (by the multiplier `r` and by the emission),
+    no exponential and no logarithm.  Every eighth step the largest element of the new state vector is looked
+    up; the vector itself is left alone and the next step multiplies what it produces by a power of two that
+    brings that element back to just under one (the step is linear, so this is the same as scaling its input,
+    without a second pass over the vector).  A power of two scales without rounding, and all that has to be
+    remembered of it is its exponent: the running scale is an integer count of doublings, and the time loop
+    holds no float64 arithmetic at all.  The result is float64:
+    log-likelihood = log(sum of the final vector) - doublings * log(2) - len * log_emit_scale.
+
+    Range: between two look-ups the vector may shrink by up to 2^62 (the largest multiplier) and be brought
+    back in full; what shrinks faster is brought back by 2^62 each time and keeps shrinking, and an element more
+    than 2^126 below one flushes towards zero as single precision does.  A state vector that underflows
+    completely gives log(0) = -inf, as log space would."""
     parpy.label('inst')
     for inst in range(seqs["num_instances"]):
         o0 = seqs["data"][inst, 0]
         parpy.label('state')
         for state in range(hmm["num_states"]):
             beta1[inst, state] = hmm["pinit"][state] * hmm["pemit"][o0, state]
-        scale = float64(0.0)
-        tops = float64(1.0)
+        doublings = int64(0)
         r = float32(1.0)
         for t in range(1, seqs["maxlen"]):
             forward_scaled_step(hmm, seqs, beta1, beta2, inst, t, r)
@@ -401,17 +413,16 @@ def forward_scaled(hmm, seqs, result, beta1, beta2):
                 r = float32(1.0)
                 if t % 8 == 0:
                     top = forward_scaled_top(hmm, seqs, beta1, beta2, inst, t)
-                    r = float32(1.0) / top
-                    tops = tops * float64(top)
-                    if t % 64 == 0:
-                        scale = scale + log(tops)
-                        tops = float64(1.0)
+                    k = scaled_doublings(top)
+                    r = float32(int64(1) << k)
+                    doublings = doublings + k
         beta = beta1
         if seqs["lens"][inst] & 1 == 0:
             beta = beta2
         parpy.label('state')
         total = sum(beta[inst, :])
-        result[inst] = scale + log(float64(total) * float64(r) * tops) - float64(seqs["lens"][inst]) * hmm["log_emit_scale"]
+        result[inst] = (log(float64(total) * float64(r)) - float64(doublings) * float64(0.6931471805599453)
+                        - float64(seqs["lens"][inst]) * hmm["log_emit_scale"])
 
 
 # ---------------------------------------------------------------- HMM forward, reference (16-layer) model, scaled linear space
@@ -453,17 +464,16 @@ def forward_kernel_scaled(hmm, seqs, result, beta1, beta2):
     itself in the last layer).  Tables are probabilities: `ptrans1` [4^k, 4], `pdur` [16] (the reference's
     `trans2`), `pnext` [16] (1 for layers 0..13, 1 - tail for layer 14, tail for the last layer's self loop),
     `pinit`, and `pemit` [101, 4^k] = emission probabilities times exp(`log_emit_scale`).  The reference's
-    emission tables reach down to 1e-10, so the divisor is renewed every fourth step (in the way described at
-    `forward_scaled`: the largest element is looked up, the next step divides by it) and the logarithm of the
-    collected divisors is taken every 32 steps.  The result is float64, as in `forward_scaled`."""
+    emission tables reach down to 1e-10, so the multiplier is renewed every fourth step (in the way described at
+    `forward_scaled`: the largest element is looked up, the next step multiplies by the power of two that brings
+    it back to just under one, and the doublings are counted).  The result is float64, as in `forward_scaled`."""
     parpy.label('inst')
     for inst in range(seqs["num_instances"]):
         o0 = seqs["data"][inst, 0]
         parpy.label('state')
         for state in range(hmm["num_states"]):
             beta1[inst, state] = hmm["pinit"][state] * hmm["pemit"][o0, state % (hmm["num_states"] // 16)]
-        scale = float64(0.0)
-        tops = float64(1.0)
+        doublings = int64(0)
         r = float32(1.0)
         for t in range(1, seqs["maxlen"]):
             forward_kernel_scaled_step(hmm, seqs, beta1, beta2, inst, t, r)
@@ -471,17 +481,16 @@ def forward_kernel_scaled(hmm, seqs, result, beta1, beta2):
                 r = float32(1.0)
                 if t % 4 == 0:
                     top = forward_scaled_top(hmm, seqs, beta1, beta2, inst, t)
-                    r = float32(1.0) / top
-                    tops = tops * float64(top)
-                    if t % 32 == 0:
-                        scale = scale + log(tops)
-                        tops = float64(1.0)
+                    k = scaled_doublings(top)
+                    r = float32(int64(1) << k)
+                    doublings = doublings + k
         beta = beta1
         if seqs["lens"][inst] & 1 == 0:
             beta = beta2
         parpy.label('state')
         total = sum(beta[inst, :])
-        result[inst] = scale + log(float64(total) * float64(r) * tops) - float64(seqs["lens"][inst]) * hmm["log_emit_scale"]
+        result[inst] = (log(float64(total) * float64(r)) - float64(doublings) * float64(0.6931471805599453)
+                        - float64(seqs["lens"][inst]) * hmm["log_emit_scale"])
 
 
 # ---------------------------------------------------------------- seeded inputs
