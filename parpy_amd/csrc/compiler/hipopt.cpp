@@ -584,10 +584,10 @@ struct Pass {
         out.push_back(r);
         continue;
       }
-      std::set<Name> varying;
+      std::set<Name> varying, reassigned;
       visit_stmts(s->body, [&](const S& c) {
         if (c->k == Stmt::Def || c->k == Stmt::For) varying.insert(c->id);
-        if (c->k == Stmt::Assign && c->dst->k == Expr::Var) varying.insert(c->dst->name);
+        if (c->k == Stmt::Assign && c->dst->k == Expr::Var) { varying.insert(c->dst->name); reassigned.insert(c->dst->name); }
       });
       Stmts pre, body;
       for (auto& c : s->body) {
@@ -598,7 +598,7 @@ struct Pass {
         std::map<Name, E> defs;   // definitions in the body that are pure functions of the iteration
         std::function<void(const Stmts&)> collect_defs = [&](const Stmts& b) {
           for (auto& d : b) {
-            if (d->k == Stmt::Def && d->ty.is_scalar() && !has_load(d->expr)) {
+            if (d->k == Stmt::Def && d->ty.is_scalar() && !has_load(d->expr) && !reassigned.count(d->id)) {   // a name assigned again stands for several values
               E e = subst_vars(d->expr, defs);
               bool pure = true;
               visit_exprs(e, [&](const E& x) { if (x->k == Expr::Var && !iter_vars.count(x->name)) pure = false; });
@@ -2884,6 +2884,11 @@ struct PersistentLoops {
         if (it == seen.end()) { seen[q.id] = f.params.size(); f.params.push_back(q); }
         else if (!q.read_only) f.params[it->second].read_only = false;
       }
+    // What the workgroups exchange is loaded and stored at device scope, which the printer does for elements of
+    // four bytes and more; narrower elements would keep plain cached accesses and a compute unit could serve a line
+    // that another workgroup rewrote a step ago.  Such loops stay a loop of launches.
+    for (auto& q : f.params)
+      if (q.ty.k == Type::Pointer && !q.read_only && elem_bytes(q.ty.sz) < 4) return S();
     Type u32 = Type::scalar(ElemSize::U32);
     KernelParam counter, status, limit;
     counter.id = gen.fresh("parpy_bar_counter"); counter.ty = Type::pointer(ElemSize::U32);

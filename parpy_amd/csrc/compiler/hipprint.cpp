@@ -1033,11 +1033,12 @@ struct DevicePrinter {
           if (!independent(acc[member[c]], acc[j])) ok = false;
         }
       }
-      // the index of the group must not use anything defined inside the span it moves across
+      // the index of the group must not use anything defined or assigned inside the span it moves across
       if (ok) {
         std::set<Name> defined;
         for (size_t s2 = acc[first].pos; s2 <= acc[last].pos && s2 < hi; ++s2)
           if (ss[s2]->k == Stmt::Def) defined.insert(ss[s2]->id);
+          else if (ss[s2]->k == Stmt::Assign && ss[s2]->dst->k == Expr::Var) defined.insert(ss[s2]->dst->name);   // `q = q + 1` between two members: same text, other element
         visit_exprs(a0.f, [&](const E& x) { if (x->k == Expr::Var && defined.count(x->name)) ok = false; });
       }
       if (!ok) continue;

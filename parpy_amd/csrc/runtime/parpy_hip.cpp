@@ -183,9 +183,13 @@ int32_t check_barrier_status(Plan& p) {
   p.barrier_pending = false;
   unsigned status = 0;
   if (int32_t rc = check(hipMemcpy(&status, p.barrier_words + 4, sizeof status, hipMemcpyDeviceToHost), "reading the barrier status")) return rc;
-  if (status != 0)
+  if (status != 0) {
+    // the status word is only ever cleared here, after it has been reported: a later launch of the same plan
+    // finds it set, leaves at its first barrier, and cannot hide that an earlier one was cut short
+    (void)hipMemset(p.barrier_words + 4, 0, sizeof status);
     return fail("a barrier over all workgroups of a kernel that runs a whole loop of steps timed out: the workgroups "
                 "left the kernel early and its results are incomplete (PARPY_HIP_BARRIER_POLLS sets the limit)");
+  }
   return 0;
 }
 
@@ -287,7 +291,8 @@ struct PlanBuilder {
         s.fits = ok && (int64_t)per_cu * cus >= (int64_t)s.grid[0] * s.grid[1] * s.grid[2];
         if (s.fits && !p.barrier_words) {
           void* w = nullptr;
-          if (hipMalloc(&w, 8 * sizeof(unsigned)) != hipSuccess) { (void)hipGetLastError(); s.fits = false; }
+          if (hipMalloc(&w, 8 * sizeof(unsigned)) != hipSuccess) { (void)hipGetLastError(); s.fits = false; w = nullptr; }
+          else if (hipMemset(w, 0, 8 * sizeof(unsigned)) != hipSuccess) { (void)hipGetLastError(); (void)hipFree(w); s.fits = false; w = nullptr; }
           p.barrier_words = (unsigned*)w;
         }
       }
@@ -469,7 +474,9 @@ int32_t run_stmt(Plan& p, const HStmt& s) {
         ptrs[k] = &storage[k];
       }
       if (persist) {
-        if (int32_t rc = check(hipMemsetAsync(p.barrier_words, 0, 8 * sizeof(unsigned), p.launch_stream), "clearing the barrier words")) return rc;
+        // the counter (first 16 bytes) starts from zero in every launch; the status word 16 bytes on stays as it is
+        // until the host has read it
+        if (int32_t rc = check(hipMemsetAsync(p.barrier_words, 0, 4 * sizeof(unsigned), p.launch_stream), "clearing the barrier counter")) return rc;
         // polls of the counter before a workgroup gives up: about a microsecond each, two seconds by default
         unsigned limit = 1u << 21;
         if (const char* e = getenv("PARPY_HIP_BARRIER_POLLS")) limit = (unsigned)strtoul(e, nullptr, 10);

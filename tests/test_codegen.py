@@ -330,6 +330,42 @@ def test_adjacent_accesses_are_only_packed_when_nothing_they_pass_can_touch_them
     assert "const parpy_vec4<float>" not in s
 
 
+def test_accesses_whose_index_scalar_is_assigned_between_them_are_not_packed():
+    """`4 * q`, `4 * q + 1`, ... read like one group of four, but `q` is assigned a new value between the accesses:
+    each access is a different group's element and keeps its own load and store."""
+    @parpy.jit
+    def walk(a, b, N):
+        parpy.label('i')
+        for i in range(N):
+            q = i
+            x0 = a[4 * q]
+            q = q + 1
+            x1 = a[4 * q + 1]
+            q = q + 1
+            x2 = a[4 * q + 2]
+            q = q + 1
+            x3 = a[4 * q + 3]
+            b[i] = x0 + x1 + x2 + x3
+
+    @parpy.jit
+    def walk_stores(a, b, N):
+        parpy.label('i')
+        for i in range(N):
+            q = i
+            x = a[i]
+            b[4 * q] = x
+            q = q + 1
+            b[4 * q + 1] = x
+            q = q + 1
+            b[4 * q + 2] = x
+            q = q + 1
+            b[4 * q + 3] = x
+    a, b = np.zeros(8192, dtype=np.float32), np.zeros(8192, dtype=np.float32)
+    o = opts_for({'i': parpy.threads(1024)})
+    assert "pk_" not in compiles(parpy.print_compiled(walk, [a, b, 1024], o))
+    assert "pk_" not in compiles(parpy.print_compiled(walk_stores, [a, b, 1024], o))
+
+
 def _reference_format_args(k, n=4, maxlen=30, seed=5):
     """Random tables in the layout of the reference's 16-layer model, with the probability tables of the scaled form."""
     rng = np.random.default_rng(seed)
@@ -463,6 +499,30 @@ def test_persistent_loops_emit_one_kernel_for_the_host_loop_and_keep_the_loop_as
     assert re.search(r"\} else \{\n\s+for \(int64_t t_\d+ = 1; t_\d+ < 30;", host)
     s0 = compiles(parpy.print_compiled(W.forward_syn, args, opts_for({'inst': parpy.threads(4), 'state': parpy.threads(2048)})))
     assert "parpy_grid_fits_device" not in s0 and "_steps_" not in s0
+
+
+def test_persistent_loops_keep_the_loop_of_launches_for_arrays_of_narrow_elements():
+    """Workgroups exchange data through device-scope loads and stores, which exist for elements of four bytes and
+    more: a ping-pong step over float16 or int8 vectors stays a loop of launches, the float32 one becomes one kernel."""
+    @parpy.jit
+    def pingpong(a, b, N, M, T):
+        parpy.label('i')
+        for i in range(N):
+            for t in range(T):
+                src = a
+                dst = b
+                if t & 1:
+                    src = b
+                    dst = a
+                parpy.label('j')
+                for j in range(M):
+                    dst[i, j] = src[i, (j + 1) % M] + src[i, j]
+    for dt, fused in ((np.float32, True), (np.float16, False), (np.int8, False), (np.int32, True)):
+        a = np.zeros((2, 4096), dtype=dt)
+        s = compiles(parpy.print_compiled(pingpong, [a, a.copy(), 2, 4096, 10],
+                                          opts_for({'i': parpy.threads(2), 'j': parpy.threads(4096).tpb(256)}, persistent_loops=True)))
+        assert ("parpy_grid_fits_device" in s) == fused, dt
+        assert ("_steps_" in s) == fused, dt
 
 
 def test_hmm_multi_block_hoists_time_loop_to_host():

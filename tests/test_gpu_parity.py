@@ -1083,3 +1083,14 @@ def test_persistent_step_loop_reports_a_barrier_that_times_out(monkeypatch):
     parpy.sync(HIP)
     want = oracle.hmm_syn_forward(hmm, seqs, np.float32)
     assert np.allclose(res.cpu().numpy(), want, atol=1e-5, rtol=1e-5)
+    # a run that was cut short followed, without a synchronisation in between, by a run with the normal limit: the
+    # second launch must not wipe out the first one's report
+    monkeypatch.setenv("PARPY_HIP_BARRIER_POLLS", "0")
+    W.forward_syn(hd, sd, res, a1, a2, opts=o)
+    monkeypatch.delenv("PARPY_HIP_BARRIER_POLLS")
+    W.forward_syn(hd, sd, res, a1, a2, opts=o)
+    with pytest.raises(RuntimeError, match="barrier over all workgroups .* timed out"):
+        parpy.sync(HIP)
+    W.forward_syn(hd, sd, res, a1, a2, opts=o)
+    parpy.sync(HIP)
+    assert np.allclose(res.cpu().numpy(), want, atol=1e-5, rtol=1e-5)

@@ -276,3 +276,51 @@ def test_strided_programs_on_device(case):
             parpy.jit(f)(*got, N, opts=o)
             # (products and sums may be contracted into fused multiply-adds on the device: not bit-equal)
             assert np.allclose(got[-1], want[-1], rtol=1e-5, atol=1e-6), (src, T, per, tpb, share, narrow, np.abs(got[-1] - want[-1]).max())
+
+
+# ---------------------------------------------------------------- index scalars that are assigned again between accesses
+def walking_program(rng, case):
+    """Groups of four accesses whose subscripts read alike (`4 * q + c`) while `q` moves between them, on loads, on
+    stores, or on both: every access has to keep the element that the sequential program names."""
+    name = f"walking_{case}"
+    steps = [int(rng.integers(0, 3)) for _ in range(3)]          # how far q moves after each access (0: stays)
+    loads = case % 3 != 1
+    stores = case % 3 != 0
+    lines = [f"def {name}(a, b, N):", "    parpy.label('i')", "    for i in range(N):", "        q = i"]
+    for c in range(4):
+        src = f"a[4 * q + {c}]" if loads else f"a[4 * i + {c}]"
+        dst = f"b[4 * q + {c}]" if stores else f"b[4 * i + {c}]"
+        lines.append(f"        x{c} = {src} + {c}.0")
+        lines.append(f"        {dst} = x{c}")
+        if c < 3 and steps[c]:
+            lines.append(f"        q = q + {steps[c]}")
+    return name, "\n".join(lines) + "\n"
+
+
+WALKING = list(range(9))
+
+
+@pytest.mark.parametrize("case", WALKING[:3])
+def test_walking_programs_compile(case):
+    rng = np.random.default_rng(4000 + case)
+    name, src = walking_program(rng, case)
+    f = build(name, src)
+    s = parpy.print_compiled(f, [np.zeros(4 * 300, dtype=np.float32), np.zeros(4 * 300, dtype=np.float32), 256], opts_for({'i': parpy.threads(256)}))
+    hiprtc_compile(s[:s.index("// host side")], opts_for({}))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", WALKING)
+def test_walking_programs_on_device(case):
+    rng = np.random.default_rng(4000 + case)
+    name, src = walking_program(rng, case)
+    f = build(name, src)
+    N = 256
+    # component c of an iteration goes to element 4 * (i + offset_c) + c: no two iterations store to the same element,
+    # so the parallel run has one defined result; elements nobody stores to keep the marker value
+    a = rng.uniform(-1, 1, 4 * (N + 8)).astype(np.float32)
+    want = np.full(4 * (N + 8), -7.0, dtype=np.float32)
+    f(a.copy(), want, N)
+    got = np.full(4 * (N + 8), -7.0, dtype=np.float32)
+    parpy.jit(f)(a.copy(), got, N, opts=opts_for({'i': parpy.threads(N)}))
+    assert np.array_equal(got, want), (src, np.abs(got - want).max())
