@@ -339,6 +339,68 @@ def forward_syn4(hmm, seqs, result, alpha1, alpha2):
         forward_syn_lse(hmm, seqs, result, alpha1, alpha2, inst)
 
 
+# ---------------------------------------------------------------- probability tables of the linear-space forms
+@parpy.jit
+def probability(x):
+    """exp of a single-precision logarithm, taken in double precision and rounded once."""
+    return float32(exp(float64(x)))
+
+
+@parpy.jit
+def emission_probabilities(hmm, lin, rowmax):
+    """`pemit` = exp(output_prob - emit_max) with `emit_max` the largest entry of the whole table (row maxima
+    first, then the maximum of those), so that the largest emission probability becomes one."""
+    parpy.label('obs')
+    for o in range(hmm["num_obs"]):
+        parpy.label('state')
+        rowmax[o] = max(hmm["output_prob"][o, :])
+    parpy.label('obs')
+    lin["emit_max"][0] = max(rowmax[:])
+    parpy.label('obs')
+    for o in range(hmm["num_obs"]):
+        parpy.label('state')
+        for s in range(hmm["num_kmers"]):
+            lin["pemit"][o, s] = float32(exp(float64(hmm["output_prob"][o, s]) - float64(lin["emit_max"][0])))
+
+
+@parpy.jit
+def scaled_tables(hmm, lin, rowmax):
+    """The synthetic model's log-space tables (`trans1`, `stay`, `initial_prob`, `output_prob`) as the probability
+    tables `forward_scaled` and `forward_syn4` read: `ptrans1`, `pstay`, `pinit`, `pemit`, `emit_max`."""
+    emission_probabilities(hmm, lin, rowmax)
+    parpy.label('all')
+    for s in range(hmm["num_states"]):
+        lin["pstay"][s] = probability(hmm["stay"][s])
+        lin["pinit"][s] = probability(hmm["initial_prob"][s])
+        for u in range(4):
+            lin["ptrans1"][s, u] = probability(hmm["trans1"][s, u])
+
+
+@parpy.jit
+def scaled_reference_tables(hmm, lin, rowmax):
+    """The reference's 16-layer model (tables of `load_reference_model`) as the probability tables
+    `forward_kernel_scaled` reads: `ptrans1` [4^k, 4], `pdur` [16], `pnext` [16] (one for layers 0..13, 1 - tail
+    for layer 14, tail for the last layer's self loop; tail = exp(gamma)), `pinit`, `pemit`, `emit_max`."""
+    emission_probabilities(hmm, lin, rowmax)
+    parpy.label('all')
+    for s in range(hmm["num_states"]):
+        lin["pinit"][s] = probability(hmm["initial_prob"][s])
+    parpy.label('all')
+    for q in range(hmm["num_kmers"]):
+        for u in range(4):
+            lin["ptrans1"][q, u] = probability(hmm["trans1"][q, u])
+    parpy.label('layer')
+    for l in range(16):
+        lin["pdur"][l] = probability(hmm["trans2"][l])
+        tail = exp(float64(hmm["gamma"]))
+        nxt = float64(1.0)
+        if l == 14:
+            nxt = float64(1.0) - tail
+        elif l == 15:
+            nxt = tail
+        lin["pnext"][l] = float32(nxt)
+
+
 # ---------------------------------------------------------------- HMM forward, synthetic model, scaled linear space
 @parpy.jit
 def forward_scaled_step(hmm, seqs, beta1, beta2, inst, t, r):
@@ -384,8 +446,8 @@ def scaled_doublings(top):
 def forward_scaled(hmm, seqs, result, beta1, beta2):
     """The forward pass of the synthetic model in linear space with rescaling (the classical alternative to
     log space): beta[s] holds the probability alpha[s] times a running scale.  Tables are probabilities:
-    `ptrans1`, `pstay`, `pinit`, and `pemit` = emission probabilities times the constant exp(`log_emit_scale`)
-    that makes the largest of them one.  A step is one multiplication and four multiply-adds per state for the
+    `ptrans1`, `pstay`, `pinit`, and `pemit` = emission probabilities divided by the largest of them, whose
+    logarithm is `emit_max[0]` (what `scaled_tables` makes of the log-space tables).  A step is one multiplication and four multiply-adds per state for the
     sum over its predecessors and itself and two multiplications (by the multiplier `r` and by the emission),
     no exponential and no logarithm.  Every eighth step the largest element of the new state vector is looked
     up; the vector itself is left alone and the next step multiplies what it produces by a power of two that
@@ -393,7 +455,7 @@ def forward_scaled(hmm, seqs, result, beta1, beta2):
     without a second pass over the vector).  A power of two scales without rounding, and all that has to be
     remembered of it is its exponent: the running scale is an integer count of doublings, and the time loop
     holds no float64 arithmetic at all.  The result is float64:
-    log-likelihood = log(sum of the final vector) - doublings * log(2) - len * log_emit_scale.
+    log-likelihood = log(sum of the final vector) - doublings * log(2) + len * emit_max.
 
     Range: between two look-ups the vector may shrink by up to 2^62 (the largest multiplier) and be brought
     back in full; what shrinks faster is brought back by 2^62 each time and keeps shrinking, and an element more
@@ -422,7 +484,7 @@ def forward_scaled(hmm, seqs, result, beta1, beta2):
         parpy.label('state')
         total = sum(beta[inst, :])
         result[inst] = (log(float64(total) * float64(r)) - float64(doublings) * float64(0.6931471805599453)
-                        - float64(seqs["lens"][inst]) * hmm["log_emit_scale"])
+                        + float64(seqs["lens"][inst]) * float64(hmm["emit_max"][0]))
 
 
 # ---------------------------------------------------------------- HMM forward, reference (16-layer) model, scaled linear space
@@ -463,7 +525,8 @@ def forward_kernel_scaled(hmm, seqs, result, beta1, beta2):
     for four neighbouring k-mers and four layers; a layer then adds what comes down from the layer above (from
     itself in the last layer).  Tables are probabilities: `ptrans1` [4^k, 4], `pdur` [16] (the reference's
     `trans2`), `pnext` [16] (1 for layers 0..13, 1 - tail for layer 14, tail for the last layer's self loop),
-    `pinit`, and `pemit` [101, 4^k] = emission probabilities times exp(`log_emit_scale`).  The reference's
+    `pinit`, and `pemit` [101, 4^k] = emission probabilities divided by the largest of them (`emit_max` holds its
+    logarithm; `scaled_reference_tables` makes all of them from the log-space tables).  The reference's
     emission tables reach down to 1e-10, so the multiplier is renewed every fourth step (in the way described at
     `forward_scaled`: the largest element is looked up, the next step multiplies by the power of two that brings
     it back to just under one, and the doublings are counted).  The result is float64, as in `forward_scaled`."""
@@ -490,7 +553,7 @@ def forward_kernel_scaled(hmm, seqs, result, beta1, beta2):
         parpy.label('state')
         total = sum(beta[inst, :])
         result[inst] = (log(float64(total) * float64(r)) - float64(doublings) * float64(0.6931471805599453)
-                        - float64(seqs["lens"][inst]) * hmm["log_emit_scale"])
+                        + float64(seqs["lens"][inst]) * float64(hmm["emit_max"][0]))
 
 
 # ---------------------------------------------------------------- seeded inputs
@@ -624,8 +687,47 @@ def random_reference_model(k, n_reads=100, min_len=500, max_len=1500, seed=SEED,
     return hmm, seqs
 
 
+def _table_outputs(hmm, names, new):
+    """Empty result arrays of the table kernels: `new(shape)` allocates float32 (NumPy or torch)."""
+    S = hmm["num_states"]
+    nk = hmm["output_prob"].shape[1]
+    shapes = {"emit_max": (1,), "pemit": (hmm["output_prob"].shape[0], nk), "pstay": (S,), "pinit": (S,), "ptrans1": (nk, 4),
+              "pdur": (16,), "pnext": (16,)}
+    return {k: new(shapes[k]) for k in names}
+
+
+def table_kernel_call(hmm, new, reference_format=False):
+    """(jitted function, its arguments, its options) of the table kernel for a log-space model whose arrays are
+    NumPy arrays or torch tensors; `new(shape)` allocates a float32 array of the same kind for a result."""
+    names = ("emit_max", "pemit", "pinit", "ptrans1", "pdur", "pnext") if reference_format else ("emit_max", "pemit", "pstay", "pinit", "ptrans1")
+    lin = _table_outputs(hmm, names, new)
+    src = dict(hmm)
+    src["num_obs"], src["num_kmers"] = int(hmm["output_prob"].shape[0]), int(hmm["output_prob"].shape[1])
+    rowmax = new((src["num_obs"],))
+    fn = scaled_reference_tables if reference_format else scaled_tables
+    opts = parpy.par({"obs": parpy.threads(src["num_obs"]), "state": parpy.threads(256), "all": parpy.threads(src["num_states"]),
+                      "layer": parpy.threads(16)})
+    return fn, [src, lin, rowmax], opts
+
+
+def scaled_tables_on_device(hd, reference_format=False, time_it=False):
+    """Run the table kernel for a model whose log-space tables are torch tensors on the GPU and return the model
+    dict that the linear-space forward passes take (the log-space tables stay in it).  With `time_it` the device
+    time of the call in milliseconds is returned as well."""
+    import torch
+    dev = hd["output_prob"].device
+    fn, args, opts = table_kernel_call(hd, lambda shape: torch.empty(shape, dtype=torch.float32, device=dev), reference_format)
+    fn(*args, opts=opts)
+    ms = parpy.time_call(fn, *args, opts=opts) if time_it else None
+    out = dict(hd)
+    out.update(args[1])
+    return (out, ms) if time_it else out
+
+
 def with_linear_tables(hmm):
-    """The model with its transition tables also in linear space (`ptrans1`, `pstay`), as `forward_syn4` reads them."""
+    """The model with its transition tables also in linear space (`ptrans1`, `pstay`), as `forward_syn4` reads them.
+    Host-side statement of what `scaled_tables` computes on the device: used where no GPU is there (code generation
+    tests) and as the checker of the device tables."""
     out = dict(hmm)
     out["ptrans1"] = np.exp(hmm["trans1"].astype(np.float64)).astype(np.float32)
     out["pstay"] = np.exp(hmm["stay"].astype(np.float64)).astype(np.float32)
@@ -633,19 +735,18 @@ def with_linear_tables(hmm):
 
 
 def with_scaled_tables(hmm):
-    """The model with probability tables for `forward_scaled`: `ptrans1`, `pstay`, `pinit`, and the emission
-    probabilities times one constant that makes the largest of them one (`pemit`; `log_emit_scale` is the
-    logarithm of that constant, a Python float and so a compile-time constant of the kernel)."""
+    """Host-side statement of `scaled_tables` (see `with_linear_tables`): `ptrans1`, `pstay`, `pinit`, `emit_max` =
+    the largest entry of the log-space emission table (one float32 element) and `pemit` = exp(output_prob - emit_max)."""
     out = with_linear_tables(hmm)
     out["pinit"] = np.exp(hmm["initial_prob"].astype(np.float64)).astype(np.float32)
     e = hmm["output_prob"].astype(np.float64)
-    out["log_emit_scale"] = float(-e.max())
-    out["pemit"] = np.exp(e + out["log_emit_scale"]).astype(np.float32)
+    out["emit_max"] = np.array([e.max()], dtype=np.float32)
+    out["pemit"] = np.exp(e - float(out["emit_max"][0])).astype(np.float32)
     return out
 
 
 def with_scaled_reference_tables(hmm):
-    """The reference's 16-layer model with the probability tables `forward_kernel_scaled` reads (see there)."""
+    """Host-side statement of `scaled_reference_tables` (see `with_linear_tables`)."""
     out = dict(hmm)
     out["ptrans1"] = np.exp(hmm["trans1"].astype(np.float64)).astype(np.float32)
     out["pdur"] = np.exp(hmm["trans2"].astype(np.float64)).astype(np.float32)
@@ -653,8 +754,8 @@ def with_scaled_reference_tables(hmm):
     out["pnext"] = np.array([1.0] * 14 + [1.0 - tail, tail], dtype=np.float32)
     out["pinit"] = np.exp(hmm["initial_prob"].astype(np.float64)).astype(np.float32)
     e = hmm["output_prob"].astype(np.float64)
-    out["log_emit_scale"] = float(-e.max())
-    out["pemit"] = np.exp(e + out["log_emit_scale"]).astype(np.float32)
+    out["emit_max"] = np.array([e.max()], dtype=np.float32)
+    out["pemit"] = np.exp(e - float(out["emit_max"][0])).astype(np.float32)
     return out
 
 

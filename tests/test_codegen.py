@@ -412,7 +412,7 @@ def test_what_the_iterations_of_one_thread_share_is_evaluated_once_per_thread():
     scores in the source vector (a local pointer that never names the array the loop stores to) and the emission
     depend on g alone and are loaded in front of the counted loop; `state // 4096` is the counter itself."""
     args = _reference_format_args(6, n=2, maxlen=6)
-    hmm = {k: v for k, v in args[0].items() if not k.startswith("p") and k != "log_emit_scale"}
+    hmm = {k: v for k, v in args[0].items() if not k.startswith("p") and k != "emit_max"}
     a = np.zeros((2, hmm["num_states"]), dtype=np.float32)
     call = [hmm, args[1], a, a.copy(), np.zeros(2, dtype=np.float32)]
     o = opts_for({'inst': parpy.threads(2), 'state': parpy.threads(4096)})

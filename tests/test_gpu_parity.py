@@ -266,7 +266,7 @@ def test_reference_format_models_with_random_tables(k, threads):
 
 
 def _run_reference_scaled(hmm, seqs, threads, **kw):
-    hd, sd = W.to_device(W.with_scaled_reference_tables(hmm)), W.to_device(seqs)
+    hd, sd = W.scaled_tables_on_device(W.to_device(hmm), reference_format=True), W.to_device(seqs)
     n, S = seqs["num_instances"], hmm["num_states"]
     b1 = torch.zeros((n, S), dtype=torch.float32, device="cuda")
     b2 = torch.zeros_like(b1)
@@ -362,9 +362,30 @@ def test_forward_synthetic_each_memory_pass_preserves_results(flags):
     assert np.allclose(got, base, atol=1e-3, rtol=0)
 
 
+@pytest.mark.parametrize("k", [3, 5, 7])
+def test_probability_tables_made_on_the_device(k):
+    """The compiled table kernels against their host statement: exponentials taken in double precision and rounded
+    once on both sides, so at most one unit in the last place apart; the emission maximum is exact."""
+    hmm, _ = W.synthetic_hmm(k, n_inst=2, min_len=4, max_len=8)
+    got = W.scaled_tables_on_device(W.to_device(hmm))
+    want = W.with_scaled_tables(hmm)
+    assert np.array_equal(got["emit_max"].cpu().numpy(), want["emit_max"])
+    for name in ("pemit", "ptrans1", "pstay", "pinit"):
+        g, w = got[name].cpu().numpy(), want[name]
+        assert g.shape == w.shape and np.all(np.abs(g - w) <= np.spacing(w)), (name, np.abs(g - w).max())
+    if k < 7:
+        ref, _ = _random_reference_model(k, n_reads=2, max_len=8, seed=k)
+        got = W.scaled_tables_on_device(W.to_device(ref), reference_format=True)
+        want = W.with_scaled_reference_tables(ref)
+        assert np.array_equal(got["emit_max"].cpu().numpy(), want["emit_max"])
+        for name in ("pemit", "ptrans1", "pdur", "pnext", "pinit"):
+            g, w = got[name].cpu().numpy(), want[name]
+            assert g.shape == w.shape and np.all(np.abs(g - w) <= np.spacing(w)), (name, np.abs(g - w).max())
+
+
 def _run_grouped(hmm, seqs, threads, **kw):
     """`forward_syn4`: the step written over groups of four states, transition tables in linear space."""
-    hd, sd = W.to_device(W.with_linear_tables(hmm)), W.to_device(seqs)
+    hd, sd = W.scaled_tables_on_device(W.to_device(hmm)), W.to_device(seqs)
     n, S = seqs["num_instances"], hmm["num_states"]
     a1 = torch.zeros((n, S), dtype=torch.float32, device="cuda")
     a2 = torch.zeros_like(a1)
@@ -375,7 +396,7 @@ def _run_grouped(hmm, seqs, threads, **kw):
 
 def _run_scaled(hmm, seqs, threads, **kw):
     """`forward_scaled`: linear space with rescaling, float64 result."""
-    hd, sd = W.to_device(W.with_scaled_tables(hmm)), W.to_device(seqs)
+    hd, sd = W.scaled_tables_on_device(W.to_device(hmm)), W.to_device(seqs)
     n, S = seqs["num_instances"], hmm["num_states"]
     b1 = torch.zeros((n, S), dtype=torch.float32, device="cuda")
     b2 = torch.zeros_like(b1)
