@@ -19,6 +19,7 @@ SDDMM by NumPy / PyTorch library routines.  7-mer *reference-model* parity is
 unpinned: test/data/7mer-model.hdf5 is absent from the reference checkout.
 """
 import ctypes
+import hashlib
 import os
 import subprocess
 
@@ -29,13 +30,28 @@ _LIB_PATH = os.path.join(_HERE, "liboracle.so")
 _lib = None
 
 
+_GCC = ["gcc", "-O2", "-fopenmp", "-shared", "-fPIC"]
+
+
+def _source_stamp(src):
+    h = hashlib.sha256(" ".join(_GCC).encode())
+    with open(src, "rb") as f:
+        h.update(f.read())
+    return h.hexdigest()
+
+
 def build(force=False):
-    """Compile hmm_oracle.c into liboracle.so (gcc, OpenMP)."""
+    """Compile hmm_oracle.c into liboracle.so (gcc, OpenMP); rebuilt when the source's content changed."""
     src = os.path.join(_HERE, "hmm_oracle.c")
-    if force or not os.path.exists(_LIB_PATH) or \
-            os.path.getmtime(_LIB_PATH) < os.path.getmtime(src):
-        subprocess.run(["gcc", "-O2", "-fopenmp", "-shared", "-fPIC", "-o",
-                        _LIB_PATH, src, "-lm"], check=True)
+    stamp = _LIB_PATH + ".srchash"
+    current = False
+    if os.path.exists(_LIB_PATH) and os.path.exists(stamp):
+        with open(stamp) as f:
+            current = f.read().strip() == _source_stamp(src)
+    if force or not current:
+        subprocess.run(_GCC + ["-o", _LIB_PATH, src, "-lm"], check=True)
+        with open(stamp, "w") as f:
+            f.write(_source_stamp(src))
     return _LIB_PATH
 
 

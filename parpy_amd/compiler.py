@@ -10,11 +10,10 @@ like the reference does (src/utils/err.rs:79-87, src/utils/info.rs:90-121).
 import ctypes
 import linecache
 import os
-import warnings
 import pathlib
 import subprocess
 
-from . import frontend
+from . import _buildstamp, frontend
 from .options import CompileBackend, LoopPar, ElemSize
 
 CSRC = pathlib.Path(__file__).parent / "csrc" / "compiler"
@@ -25,21 +24,24 @@ SOURCES = ["ast.cpp", "front.cpp", "constfold.cpp", "specialize.cpp", "lower.cpp
 _lib = None
 
 
-def _stale():
-    deps = [CSRC / s for s in SOURCES] + list(CSRC.glob("*.hpp")) + [pathlib.Path(__file__).parent.parent / "include" / "parpy_hipc.h"]
-    return any(os.path.getmtime(LIB_PATH) < os.path.getmtime(d) for d in deps if d.exists())
+def _deps():
+    return [CSRC / s for s in SOURCES] + sorted(CSRC.glob("*.hpp")) + [pathlib.Path(__file__).parent.parent / "include" / "parpy_hipc.h"]
+
+
+def _command():
+    return ["g++", "-std=c++17", "-O2", "-fPIC", "-shared", "-Wall", "-Wno-sign-compare"]
 
 
 def build_library(force=False):
     """Compile the compiler core with g++ (no GPU toolchain needed)."""
     srcs = [CSRC / s for s in SOURCES]
-    if not force and LIB_PATH.exists() and not _stale():
+    if not force and LIB_PATH.exists() and _buildstamp.is_current(LIB_PATH, _deps(), _command()):
         return LIB_PATH
-    cmd = ["g++", "-std=c++17", "-O2", "-fPIC", "-shared", "-Wall", "-Wno-sign-compare",
-           "-o", str(LIB_PATH)] + [str(s) for s in srcs]
+    cmd = _command() + ["-o", str(LIB_PATH)] + [str(s) for s in srcs]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"Compilation of the ParPy compiler core failed:\n{r.stdout}\n{r.stderr}")
+    _buildstamp.write_stamp(LIB_PATH, _deps(), _command())
     return LIB_PATH
 
 
@@ -47,11 +49,8 @@ def _load():
     global _lib
     if _lib is not None:
         return _lib
-    # (as for the runtime library: what is built is loaded; a library older than its sources is rebuilt on request)
-    if not LIB_PATH.exists() or os.environ.get("PARPY_AMD_REBUILD") == "1":
-        build_library()
-    elif _stale():
-        warnings.warn(f"{LIB_PATH.name} is older than its sources: run __graft_entry__.build() or set PARPY_AMD_REBUILD=1", RuntimeWarning)
+    # what is built is loaded; a library that does not match its sources (by content) is rebuilt first
+    _buildstamp.ensure_current(LIB_PATH, _deps(), _command(), lambda: build_library(force=True))
     lib = ctypes.CDLL(str(LIB_PATH))
     vp, cp, i32 = ctypes.c_void_p, ctypes.c_char_p, ctypes.c_int32
     lib.parpy_hipc_parse.argtypes = [cp, ctypes.POINTER(cp), ctypes.POINTER(vp), i32, ctypes.POINTER(vp)]

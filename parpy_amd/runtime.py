@@ -3,15 +3,15 @@
 Counterpart of python/parpy/runtime.py:11-98 of the reference: declares the
 ctypes signatures of the seven runtime exports plus the hiprtc / module /
 launch-plan entry points.  The library is built ahead of time by
-`__graft_entry__.build()`; loading it never compiles anything when the built
-file is present.
+`__graft_entry__.build()`; loading it compiles nothing when the built file
+matches its sources.
 """
 import ctypes
 import os
-import warnings
 import pathlib
 import subprocess
 
+from . import _buildstamp
 from .options import CompileBackend
 
 PARPY_NATIVE_PATH = pathlib.Path(__file__).parent / "csrc" / "runtime"
@@ -20,10 +20,6 @@ HIPCC_FLAGS = ["-O2", "-fPIC", "-shared", "-std=c++17", "--offload-arch=gfx950",
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 
 libs = {}
-
-
-def _older_than(lib, deps):
-    return any(os.path.getmtime(lib) < os.path.getmtime(d) for d in deps if d.exists())
 
 
 def _runtime_deps():
@@ -37,12 +33,13 @@ def build_library(force=False):
     src = PARPY_NATIVE_PATH / "parpy_hip.cpp"
     deps = _runtime_deps()
     lib = PARPY_HIP_BASE_LIB_PATH
-    if not force and lib.exists() and not _older_than(lib, deps):
+    if not force and lib.exists() and _buildstamp.is_current(lib, deps, HIPCC_FLAGS):
         return lib
     cmd = ["hipcc"] + HIPCC_FLAGS + ["-o", str(lib), str(src), "-lhiprtc"]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"Compilation of the HIP runtime library failed.\nstdout:\n{r.stdout}\nstderr:\n{r.stderr}")
+    _buildstamp.write_stamp(lib, deps, HIPCC_FLAGS)
     return lib
 
 
@@ -97,13 +94,9 @@ def init_library(libpath):
 def load_hip_runtime_lib():
     """Load the runtime library without requiring a GPU (hiprtc compilation works on any host)."""
     if "hip-nogpu" not in libs:
-        # A library that is there is loaded as it is (a GPU machine runs what was built beforehand); one that is
-        # older than its sources is rebuilt only on request and otherwise named in a warning.
-        if not PARPY_HIP_BASE_LIB_PATH.exists() or os.environ.get("PARPY_AMD_REBUILD") == "1":
-            build_library()
-        elif _older_than(PARPY_HIP_BASE_LIB_PATH, _runtime_deps()):
-            warnings.warn(f"{PARPY_HIP_BASE_LIB_PATH.name} is older than its sources: run __graft_entry__.build() "
-                          "or set PARPY_AMD_REBUILD=1", RuntimeWarning)
+        # what is built is loaded; a library that does not match its sources (by content, not by file time) is
+        # rebuilt first, so that a forgotten build step cannot put old code under test
+        _buildstamp.ensure_current(PARPY_HIP_BASE_LIB_PATH, _runtime_deps(), HIPCC_FLAGS, lambda: build_library(force=True))
         libs["hip-nogpu"] = init_library(PARPY_HIP_BASE_LIB_PATH)
     return libs["hip-nogpu"]
 

@@ -56,20 +56,38 @@ def test_plan_rejects_malformed_text_and_wrong_arity():
     assert lib.parpy_hip_plan_destroy(plan) == 0
 
 
-def test_a_library_older_than_its_sources_is_loaded_with_a_warning_and_rebuilt_only_on_request(monkeypatch):
-    from parpy_amd import runtime
+def test_a_library_that_does_not_match_its_sources_is_rebuilt_on_load(monkeypatch, tmp_path):
+    """Staleness goes by content (a stamp with the hash of the sources written at build time), not by file
+    times, which do not survive copying the tree: a library whose stamp differs is rebuilt with a warning,
+    PARPY_AMD_REBUILD=0 loads it as it is, and a matching one is loaded silently."""
+    import warnings
+    from parpy_amd import runtime, _buildstamp
     built = []
-    monkeypatch.setattr(runtime, "_older_than", lambda lib, deps: True)
     monkeypatch.setattr(runtime, "build_library", lambda force=False: built.append(force))
-    monkeypatch.delitem(runtime.libs, "hip-nogpu", raising=False)
     monkeypatch.delenv("PARPY_AMD_REBUILD", raising=False)
-    with pytest.warns(RuntimeWarning, match="older than its sources"):
-        assert runtime.load_hip_runtime_lib() is not None
-    assert built == []
     monkeypatch.delitem(runtime.libs, "hip-nogpu", raising=False)
-    monkeypatch.setenv("PARPY_AMD_REBUILD", "1")
-    runtime.load_hip_runtime_lib()
-    assert built == [False]
+    with warnings.catch_warnings():
+        warnings.simplefilter("error")
+        assert runtime.load_hip_runtime_lib() is not None      # as built: no warning, no compilation
+    assert built == []
+    monkeypatch.setattr(_buildstamp, "source_hash", lambda paths, command: "another hash")
+    monkeypatch.delitem(runtime.libs, "hip-nogpu", raising=False)
+    with pytest.warns(RuntimeWarning, match="does not match its sources: rebuilding"):
+        runtime.load_hip_runtime_lib()
+    assert built == [True]
+    monkeypatch.delitem(runtime.libs, "hip-nogpu", raising=False)
+    monkeypatch.setenv("PARPY_AMD_REBUILD", "0")
+    with pytest.warns(RuntimeWarning, match="PARPY_AMD_REBUILD=0 keeps it"):
+        runtime.load_hip_runtime_lib()
+    assert built == [True]
+    # the hash covers contents and the command line
+    a = tmp_path / "a.cpp"
+    a.write_text("int x;")
+    monkeypatch.undo()
+    h1 = _buildstamp.source_hash([a], ["cc"])
+    assert h1 == _buildstamp.source_hash([a], ["cc"]) and h1 != _buildstamp.source_hash([a], ["cc", "-O2"])
+    a.write_text("int y;")
+    assert h1 != _buildstamp.source_hash([a], ["cc"])
 
 
 def test_running_without_a_device_fails_loudly():
