@@ -81,6 +81,29 @@ def sddmm_csr(A, B, C, D, N, alpha, beta):
         D[i] = alpha * t + beta * C["values"][i]
 
 
+@parpy.jit
+def sddmm_coo_bt(A, BT, C, D, alpha, beta):
+    """The same product for a caller that holds B transposed (BT[j, :] = B[:, j], e.g. a constant matrix turned
+    round once): both operands of a non-zero are rows, nothing is staged per call."""
+    parpy.label('nnz')
+    for i in range(C["nnz"]):
+        row = C["rows"][i]
+        col = C["cols"][i]
+        t = sum(A[row, :] * BT[col, :])
+        D[i] = alpha * t + beta * C["values"][i]
+
+
+@parpy.jit
+def gather_row_sums(table, idx, out, n):
+    """out[i] = sum(table[idx[i], :]): one dependent index load, then a row of contiguous 128-byte lines from a
+    random place of the table, for every i -- the access pattern of SDDMM's row of B^T without the arithmetic
+    (the measure of how fast random lines come out of L2)."""
+    parpy.label('i')
+    for i in range(n):
+        r = idx[i]
+        out[i] = sum(table[r, :])
+
+
 # ---------------------------------------------------------------- HMM forward, reference (16-layer) model
 @parpy.jit
 def forward_kernel(hmm, seqs, alpha1, alpha2, result):
@@ -457,10 +480,13 @@ def forward_scaled(hmm, seqs, result, beta1, beta2):
     holds no float64 arithmetic at all.  The result is float64:
     log-likelihood = log(sum of the final vector) - doublings * log(2) + len * emit_max.
 
-    Range: between two look-ups the vector may shrink by up to 2^62 (the largest multiplier) and be brought
-    back in full; what shrinks faster is brought back by 2^62 each time and keeps shrinking, and an element more
-    than 2^126 below one flushes towards zero as single precision does.  A state vector that underflows
-    completely gives log(0) = -inf, as log space would."""
+    Range: between two look-ups (eight steps; the first window also carries the 1 / num_states of the start
+    vector) the largest element may shrink by up to 2^100, i.e. the steps of a window may on average keep as
+    little as 2^-12.5 = 1.7e-4 of the vector, measured against the most probable emission.  Within that range the
+    elements that matter (within 2^-24 of the largest) stay normal single-precision numbers and the result is
+    good to 1e-4; a multiplier is at most 2^62, what it leaves is made up at the next look-ups.  A read that
+    leaves the range (largest element positive but below 2^-100 at a look-up) gives NaN, not digits that mean
+    nothing; a read of probability zero gives log(0) = -inf, as log space would."""
     parpy.label('inst')
     for inst in range(seqs["num_instances"]):
         o0 = seqs["data"][inst, 0]
@@ -478,6 +504,8 @@ def forward_scaled(hmm, seqs, result, beta1, beta2):
                     k = scaled_doublings(top)
                     r = float32(int64(1) << k)
                     doublings = doublings + k
+                    if top > float32(0.0) and top < float32(7.888609e-31):
+                        r = (top - top) / (top - top)   # out of range (see the docstring): not a number, rather than digits that mean nothing
         beta = beta1
         if seqs["lens"][inst] & 1 == 0:
             beta = beta2
@@ -547,6 +575,8 @@ def forward_kernel_scaled(hmm, seqs, result, beta1, beta2):
                     k = scaled_doublings(top)
                     r = float32(int64(1) << k)
                     doublings = doublings + k
+                    if top > float32(0.0) and top < float32(7.888609e-31):
+                        r = (top - top) / (top - top)   # out of range (see the docstring): not a number, rather than digits that mean nothing
         beta = beta1
         if seqs["lens"][inst] & 1 == 0:
             beta = beta2

@@ -506,6 +506,50 @@ def test_forward_scaled_unreachable_and_improbable_states():
     assert np.all(np.isneginf(got) | np.isnan(got))
 
 
+def _two_symbol_model(k, log2_ratio, n_inst=4, length=100, seed=3):
+    """A synthetic model whose emission table has the same value in every state: symbol 0 with probability 1/2 and
+    symbol 1 with 2^log2_ratio of that (symbol 2: probability zero).  Every step of a read of ones keeps exactly
+    2^log2_ratio of the vector, measured against the most probable emission, and -- the transitions conserving
+    the total -- the log-likelihood of a read is the sum of the logarithms of its emissions."""
+    hmm, seqs = W.synthetic_hmm(k, n_inst=n_inst, min_len=length, max_len=length, seed=seed)
+    S = hmm["num_states"]
+    table = np.full((101, S), -np.inf, dtype=np.float32)
+    table[0, :] = np.log(0.5)
+    table[1, :] = np.log(0.5) + log2_ratio * np.log(2.0)
+    hmm["output_prob"] = table
+    rng = np.random.default_rng(seed)
+    seqs["data"] = rng.integers(0, 2, size=seqs["data"].shape).astype(np.int8)
+    seqs["data"][0, :] = 1                       # the read that shrinks at every step
+    closed = np.array([table[seqs["data"][i, :seqs["lens"][i]].astype(int), 0].astype(np.float64).sum() for i in range(n_inst)])
+    return hmm, seqs, closed
+
+
+def test_forward_scaled_at_the_edge_of_its_range():
+    """The rescaled linear-space form at the edge of what its docstring promises: a read whose every step keeps
+    2^-10 of the vector (2^-96 over the first window with its 1/64 of the start vector) is within 1e-4 of the
+    closed form and of the fp64 oracle; one whose steps keep 2^-13 leaves the range at the first look-up and gives
+    NaN, not a finite number; a read that contains an observation of probability zero gives -inf."""
+    hmm, seqs, closed = _two_symbol_model(3, -10.0)
+    want = oracle.hmm_syn_forward(hmm, seqs, np.float64)
+    assert np.abs(want - closed).max() < 1e-6 * np.abs(closed).max()
+    got = _run_scaled(hmm, seqs, 64)
+    assert np.all(np.isfinite(got)) and np.abs(got - want).max() < 1e-4, (got, want)
+    hmm, seqs, closed = _two_symbol_model(3, -13.0)
+    got = _run_scaled(hmm, seqs, 64)
+    assert np.isnan(got[0])                                       # the read of ones: out of range, and says so
+    # (reads that mix both symbols may or may not stay in range; those that are finite must be right)
+    fin = np.isfinite(got)
+    assert np.abs(got[fin] - closed[fin]).max() < 1e-4 if fin.any() else True
+    hmm, seqs, closed = _two_symbol_model(3, -3.0)
+    seqs["data"][1, 40] = 2                                        # probability zero in every state
+    want = oracle.hmm_syn_forward(hmm, seqs, np.float64)
+    got = _run_scaled(hmm, seqs, 64)
+    # (the log-space oracle ends in NaN there, like the reference's kernel: -inf - (-inf) in its closing log-sum-exp)
+    assert not np.isfinite(want[1]) and np.isneginf(got[1])
+    keep = np.arange(len(got)) != 1
+    assert np.abs(got[keep] - want[keep]).max() < 1e-4
+
+
 def test_forward_7mer_constant_emissions_closed_form():
     """Constant emissions: the log-likelihood is len * c whatever the transitions are (full headline shape)."""
     c = np.float32(np.log(1.0 / 101.0))

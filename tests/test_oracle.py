@@ -169,3 +169,27 @@ def test_product_side_model_loader_agrees_with_the_oracle(golden_dir):
             assert sorted(da) == sorted(db)
             for key in da:
                 assert np.array_equal(np.asarray(da[key]), np.asarray(db[key])), (k, key)
+
+
+def test_synthetic_forward_with_state_independent_emissions_and_an_impossible_observation():
+    """Emissions that do not depend on the state: the transitions conserve the total probability, so the
+    log-likelihood is the sum of the emission logarithms of the read.  An observation of probability zero in every
+    state makes every score -inf; the closing log-sum-exp of the reference's kernel then computes -inf - (-inf) and
+    ends in NaN (test/test_forward.py:155-160 has no repair there, unlike the step), which the oracle reproduces."""
+    from parpy_amd import workloads as W
+    hmm, seqs = W.synthetic_hmm(3, n_inst=3, min_len=40, max_len=40, seed=5)
+    S = hmm["num_states"]
+    table = np.full((101, S), -np.inf, dtype=np.float32)
+    table[0, :] = np.log(0.5)
+    table[1, :] = np.log(0.5) - 7.0
+    hmm["output_prob"] = table
+    rng = np.random.default_rng(5)
+    seqs["data"] = rng.integers(0, 2, size=seqs["data"].shape).astype(np.int8)
+    closed = np.array([table[seqs["data"][i].astype(int), 0].astype(np.float64).sum() for i in range(3)])
+    for prec, tol in ((np.float64, 1e-9), (np.float32, 1e-3)):
+        got = oracle.hmm_syn_forward(hmm, seqs, prec)
+        assert np.abs(got - closed).max() < tol * np.abs(closed).max()
+    seqs["data"][2, 17] = 2
+    for prec in (np.float64, np.float32):
+        got = oracle.hmm_syn_forward(hmm, seqs, prec)
+        assert np.isnan(got[2]) and np.all(np.isfinite(got[:2]))
