@@ -303,10 +303,21 @@ struct Restructure {
   }
 
   // ---- 5. split kernels at the remaining grid-wide synchronisation points (inter_block.rs:639-678)
+  // A nested parallel loop that is cut into several pieces takes its enclosing loops with it: the grid-wide
+  // synchronisation between two pieces (a multi-block reduction under two parallel levels: partial results per
+  // block, then their reduction) is repeated one level up, where it cuts the enclosing loop in the same place, so
+  // that the first kernel maps (outer loops, blocks, threads) and the second (outer loops, threads).
+  void push_pieces(Stmts& body, const S& child, const Stmts& pieces) {
+    for (size_t k = 0; k < pieces.size(); ++k) {
+      body.push_back(pieces[k]);
+      if (k + 1 < pieces.size() && child->par.is_parallel()) body.push_back(mk_syncpoint(SyncKind::InterBlock, child->i));
+    }
+  }
+
   Stmts split_kernel(const S& loop) {
     Stmts body;
     for (auto& s : loop->body) {
-      if (s->k == Stmt::For) for (auto& r : split_kernel(s)) body.push_back(r);
+      if (s->k == Stmt::For) push_pieces(body, s, split_kernel(s));
       else if (!s->body.empty() || !s->els.empty()) {
         auto r = clone(s);
         r->body = split_in_kernel(s->body);
@@ -322,7 +333,7 @@ struct Restructure {
   Stmts split_in_kernel(const Stmts& ss) {
     Stmts out;
     for (auto& s : ss) {
-      if (s->k == Stmt::For) for (auto& r : split_kernel(s)) out.push_back(r);
+      if (s->k == Stmt::For) push_pieces(out, s, split_kernel(s));
       else if (!s->body.empty() || !s->els.empty()) {
         auto r = clone(s);
         r->body = split_in_kernel(s->body);

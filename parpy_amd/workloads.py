@@ -461,8 +461,14 @@ def forward_scaled_top(hmm, seqs, beta1, beta2, inst, t):
 @parpy.jit
 def scaled_doublings(top):
     """How many times the state vector whose largest element is `top` can be doubled without passing one
-    (0 .. 62; nothing has to be exact here, any power of two near 1 / top serves as the divisor)."""
-    return int64(min(max(-log(top) * float32(1.4426950408889634), float32(0.0)), float32(62.0)))
+    (0 .. 120; nothing has to be exact here, any power of two near 1 / top serves as the multiplier)."""
+    return int64(min(max(-log(top) * float32(1.4426950408889634), float32(0.0)), float32(120.0)))
+
+
+@parpy.jit
+def power_of_two(k):
+    """2^k in single precision for 0 <= k <= 120, exactly: the product of two shifted ones."""
+    return float32(int64(1) << min(k, int64(60))) * float32(int64(1) << max(k - int64(60), int64(0)))
 
 
 @parpy.jit
@@ -484,7 +490,7 @@ def forward_scaled(hmm, seqs, result, beta1, beta2):
     vector) the largest element may shrink by up to 2^100, i.e. the steps of a window may on average keep as
     little as 2^-12.5 = 1.7e-4 of the vector, measured against the most probable emission.  Within that range the
     elements that matter (within 2^-24 of the largest) stay normal single-precision numbers and the result is
-    good to 1e-4; a multiplier is at most 2^62, what it leaves is made up at the next look-ups.  A read that
+    good to 1e-4.  A read that
     leaves the range (largest element positive but below 2^-100 at a look-up) gives NaN, not digits that mean
     nothing; a read of probability zero gives log(0) = -inf, as log space would."""
     parpy.label('inst')
@@ -502,7 +508,7 @@ def forward_scaled(hmm, seqs, result, beta1, beta2):
                 if t % 8 == 0:
                     top = forward_scaled_top(hmm, seqs, beta1, beta2, inst, t)
                     k = scaled_doublings(top)
-                    r = float32(int64(1) << k)
+                    r = power_of_two(k)
                     doublings = doublings + k
                     if top > float32(0.0) and top < float32(7.888609e-31):
                         r = (top - top) / (top - top)   # out of range (see the docstring): not a number, rather than digits that mean nothing
@@ -573,7 +579,7 @@ def forward_kernel_scaled(hmm, seqs, result, beta1, beta2):
                 if t % 4 == 0:
                     top = forward_scaled_top(hmm, seqs, beta1, beta2, inst, t)
                     k = scaled_doublings(top)
-                    r = float32(int64(1) << k)
+                    r = power_of_two(k)
                     doublings = doublings + k
                     if top > float32(0.0) and top < float32(7.888609e-31):
                         r = (top - top) / (top - top)   # out of range (see the docstring): not a number, rather than digits that mean nothing

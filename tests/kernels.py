@@ -80,6 +80,59 @@ def min_2d(x, out, N):
     out[0] = min(x[:, :])
 
 
+def sum_planes(x, out, N, M):
+    parpy.label('N')
+    for i in range(N):
+        parpy.label('M')
+        for j in range(M):
+            parpy.label('K')
+            out[i, j] = sum(x[i, j, :])
+
+
+def prod_planes(x, out, N, M):
+    parpy.label('N')
+    for i in range(N):
+        parpy.label('M')
+        for j in range(M):
+            parpy.label('K')
+            out[i, j] = prod(x[i, j, :])
+
+
+def max_planes(x, out, N, M):
+    parpy.label('N')
+    for i in range(N):
+        parpy.label('M')
+        for j in range(M):
+            parpy.label('K')
+            out[i, j] = max(x[i, j, :])
+
+
+def min_planes(x, out, N, M):
+    parpy.label('N')
+    for i in range(N):
+        parpy.label('M')
+        for j in range(M):
+            parpy.label('K')
+            out[i, j] = min(x[i, j, :])
+
+
+def scaled_row_sums(x, y, out, N, M):
+    """A reduction between two element-wise loops of the same nest: the row is scaled in place, summed (over more
+    threads than a workgroup holds when the options say so) and divided by its sum."""
+    parpy.label('N')
+    for i in range(N):
+        parpy.label('M')
+        for j in range(M):
+            y[i, j] = x[i, j] * 2.0 + 1.0
+        parpy.label('M')
+        s = sum(y[i, :])
+        out[i] = s
+        parpy.label('M')
+        for j in range(M):
+            y[i, j] = y[i, j] / s
+
+
+PLANE_REDUCTIONS = [sum_planes, prod_planes, max_planes, min_planes]
 ROW_REDUCTIONS = [sum_rows, prod_rows, max_rows, min_rows, sum_axis, prod_axis, max_axis, min_axis]
 FULL_REDUCTIONS = [sum_2d, prod_2d, max_2d, min_2d]
 NUMPY_OP = {"sum": "sum", "prod": "prod", "max": "max", "min": "min"}

@@ -56,6 +56,35 @@ def test_reduction_grids(fn):
     assert "parpy_alloc_buffer(3200)" in s3 and "parpy_free_buffer" in s3
 
 
+@pytest.mark.parametrize("fn", K.PLANE_REDUCTIONS)
+def test_multi_block_reductions_under_two_parallel_levels(fn):
+    """out[i, j] = op(x[i, j, :]) with more threads on the innermost level than a workgroup holds: the reduction is
+    split into partial results per block and their reduction, and the grid-wide synchronisation between the two cuts
+    both enclosing loops, so the first kernel maps (N, M, blocks, threads) and the second (N, M, threads)."""
+    N, M, K_ = 10, 20, 5000
+    x = np.zeros((N, M, K_), dtype=np.float32)
+    out = np.zeros((N, M), dtype=np.float32)
+    s = compiles(parpy.print_compiled(fn, [x, out, N, M], opts_for({'N': parpy.threads(N), 'M': parpy.threads(M), 'K': parpy.threads(2048)})))
+    assert launch(s) == [("10", "2", "20", "1024", "1", "1"), ("1", "20", "10", "64", "1", "1")]
+    assert "parpy_alloc_buffer(1600)" in s                            # 10 x 20 x 2 partial results
+    s = compiles(parpy.print_compiled(fn, [x, out, N, M], opts_for({'N': parpy.threads(N), 'M': parpy.threads(M), 'K': parpy.threads(1024).tpb(128)})))
+    assert launch(s) == [("10", "8", "20", "128", "1", "1"), ("1", "20", "10", "64", "1", "1")]
+    assert "parpy_alloc_buffer(6400)" in s
+    # within one workgroup nothing is cut
+    s = compiles(parpy.print_compiled(fn, [x, out, N, M], opts_for({'N': parpy.threads(N), 'M': parpy.threads(M), 'K': parpy.threads(256)})))
+    assert launch(s) == [("1", "20", "10", "256", "1", "1")]
+
+
+def test_multi_block_reduction_between_two_loops_of_one_nest():
+    """Element-wise loop, multi-block sum, element-wise loop that uses the sum, all under one parallel loop: four
+    kernels (scale, partial sums, their sum, divide), the sum handed on through device temporaries."""
+    N, M = 6, 4096
+    x = np.zeros((N, M), dtype=np.float32)
+    o = opts_for({'N': parpy.threads(N), 'M': parpy.threads(2048).tpb(256)})
+    s = compiles(parpy.print_compiled(K.scaled_row_sums, [x, x.copy(), np.zeros(N, dtype=np.float32), N, M], o))
+    assert [l[:3] for l in launch(s)] == [("8", "6", "1"), ("1", "8", "6"), ("1", "6", "1"), ("8", "6", "1")]
+
+
 @pytest.mark.parametrize("fn", K.FULL_REDUCTIONS)
 def test_full_reduction_compiles(fn):
     x = np.zeros((100, 50), dtype=np.float32)

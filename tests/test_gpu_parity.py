@@ -70,6 +70,36 @@ def test_reductions(fn, case):
     assert np.allclose(out, want, atol=tol, rtol=1e-5), (np.abs(out - want).max(), fn.__name__, case[0])
 
 
+@pytest.mark.parametrize("fn", K.PLANE_REDUCTIONS, ids=lambda f: f.__name__)
+@pytest.mark.parametrize("inner", [("one workgroup", lambda: parpy.threads(256)), ("2 blocks", lambda: parpy.threads(2048)),
+                                   ("8 blocks of 128", lambda: parpy.threads(1024).tpb(128))], ids=lambda c: c[0])
+def test_reductions_under_two_parallel_levels(fn, inner):
+    """sum / prod / max / min over the last axis of a 10 x 20 x 5000 array, the innermost level within one workgroup
+    and across several (partial results per block in a device temporary, a second kernel reduces them)."""
+    rng = np.random.default_rng(77)
+    N, M, K_ = 10, 20, 5000
+    x = rng.standard_normal((N, M, K_)).astype(np.float32)
+    if fn.__name__.startswith("prod"):
+        x = (1.0 + 0.001 * x).astype(np.float32)
+    out = np.zeros((N, M), dtype=np.float32)
+    parpy.jit(fn)(x, out, N, M, opts=opts_for({'N': parpy.threads(N), 'M': parpy.threads(M), 'K': inner[1]()}))
+    f = {"sum": np.sum, "prod": np.prod, "max": np.max, "min": np.min}[fn.__name__.split("_")[0]]
+    want = f(x.astype(np.float64), axis=2).astype(np.float32)
+    assert np.allclose(out, want, atol=1e-4, rtol=1e-5), (fn.__name__, inner[0], np.abs(out - want).max())
+
+
+@pytest.mark.parametrize("inner", [("one workgroup", lambda: parpy.threads(512)), ("8 blocks of 256", lambda: parpy.threads(2048).tpb(256))], ids=lambda c: c[0])
+def test_reduction_between_two_loops_of_one_nest(inner):
+    rng = np.random.default_rng(78)
+    N, M = 6, 4096
+    x = rng.uniform(0.0, 1.0, (N, M)).astype(np.float32)
+    y, out = np.zeros_like(x), np.zeros(N, dtype=np.float32)
+    parpy.jit(K.scaled_row_sums)(x, y, out, N, M, opts=opts_for({'N': parpy.threads(N), 'M': inner[1]()}))
+    t = x.astype(np.float64) * 2.0 + 1.0
+    assert np.allclose(out, t.sum(axis=1), rtol=1e-5), np.abs(out - t.sum(axis=1)).max()
+    assert np.allclose(y, t / t.sum(axis=1, keepdims=True), rtol=1e-5, atol=1e-9)
+
+
 @pytest.mark.parametrize("lane_split", [True, False])
 def test_one_thread_per_row_on_many_rows(lane_split):
     """4096 rows summed by one thread each: eight lanes share a row when the lane-group pass is on."""
