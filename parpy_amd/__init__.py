@@ -91,10 +91,56 @@ def _compile_function(ir_ast, args, opts):
     top_map = _callable_names(opts.backend)
     res = compiler.compile_ir(ir_ast, args, opts, top_map)
     cache_key = _generate_function_key(res.device_src, opts)
-    build_code_object(cache_key, res.device_src, opts)
+    path = build_code_object(cache_key, res.device_src, opts)
+    res, cache_key = _register_feedback(ir_ast, args, opts, top_map, name, res, cache_key, path)
     wrap_fn = get_wrapper(name, cache_key, res.plan, opts)
     _fun_cache[fast_cache_key] = wrap_fn
     return wrap_fn
+
+
+def _register_feedback(ir_ast, args, opts, top_map, name, res, cache_key, path):
+    """The register budgets of the caching passes are estimates; the compiled code object says how they turned
+    out.  When it reports spilled vector registers (and the budget was not set by hand) the function is
+    compiled again with 80 % and, if that still spills, 60 % of the budget, and the version that spills the least
+    is kept.  With `opts.reg_feedback_timed` the choice is made by the clock instead: the versions for 100, 80, 60,
+    45 and 30 % of the budget (those that differ) are each run and timed on the arguments of this call and the
+    fastest is kept -- which executes the function several times, so only for functions whose result does not
+    depend on how often they ran."""
+    from .codeobject import spilled_vgprs
+    from .compile import build_code_object, get_wrapper
+    from .key import _generate_function_key
+    import copy
+    if not (opts.reg_feedback or opts.reg_feedback_timed) or opts.reg_budget is not None or opts.reg_budget_scale is not None:
+        return res, cache_key
+    with open(path, "rb") as f:
+        spills = spilled_vgprs(f.read())
+    if spills == 0 and not opts.reg_feedback_timed:
+        return res, cache_key
+    candidates = [(spills, 100, res, cache_key)]
+    seen = {res.device_src}
+    for scale in ((80, 60, 45, 30) if opts.reg_feedback_timed else (80, 60)):
+        o2 = copy.copy(opts)
+        o2.reg_budget_scale = scale
+        r2 = compiler.compile_ir(ir_ast, args, o2, top_map)
+        if r2.device_src in seen:      # the budget does not bind: nothing the passes decide changes the code
+            continue
+        seen.add(r2.device_src)
+        k2 = _generate_function_key(r2.device_src, o2)
+        with open(build_code_object(k2, r2.device_src, o2), "rb") as f:
+            s2 = spilled_vgprs(f.read())
+        candidates.append((s2, scale, r2, k2))
+        if s2 == 0 and not opts.reg_feedback_timed:
+            break
+    if opts.reg_feedback_timed and len(candidates) > 1:
+        times = []
+        for c in candidates:
+            w = get_wrapper(name, c[3], c[2].plan, opts)
+            w.timed(*args)
+            times.append(min(w.timed(*args) for _ in range(2)))
+        best = candidates[times.index(min(times))]
+    else:
+        best = min(candidates, key=lambda c: (c[0], -c[1]))
+    return best[2], best[3]
 
 
 def threads(n):

@@ -213,6 +213,8 @@ def describe_opts(opts):
             parts.append(f"({name} {1 if v else 0})")
     if getattr(opts, "reg_budget", None):
         parts.append(f"(reg_budget {int(opts.reg_budget)})")
+    if getattr(opts, "reg_budget_scale", None):
+        parts.append(f"(reg_budget_scale {int(opts.reg_budget_scale)})")
     return f"(opts {' '.join(parts)})"
 
 

@@ -391,6 +391,7 @@ struct Options {  // src/option.rs:14-108
   bool opt_fence_iterations = true;   // the unrolled iterations of a thread that read and write LDS are scheduled one after the other
   bool opt_expand_short_loops = true; // counted loops of <= 8 iterations inside a parallel iteration are expanded in place
   int64_t reg_budget = 0;     // 32-bit registers per thread the caching passes may claim (0 = by block size)
+  int64_t reg_budget_scale = 100;   // percent of the by-block-size budget (the driver lowers it when a code object spills)
   bool assume_aligned = true;  // array arguments are at least 16-byte aligned
   ElemSize int_size() const { return has_force_int ? force_int : ElemSize::I64; }
   ElemSize float_size() const { return has_force_float ? force_float : ElemSize::F64; }

@@ -1275,9 +1275,13 @@ struct Pass {
     int64_t threads = k.block.x * k.block.y * k.block.z;
     // a 1024-thread block leaves 128 VGPRs per lane; 88 cached values plus the
     // working set fit without spilling (measured on the HMM kernels; 96 spills a few)
-    if (threads <= 512) return threads <= 256 ? 192 : 128;
-    // a per-element step body without exponentials or logarithms keeps few values alive besides the cached ones
-    return step_has_transcendentals() ? 88 : 104;
+    // (workgroups of up to 512 threads leave a wave 256 registers or more: 192 cached values and the working set fit;
+    // with 128 the 7-mer HMM forms on 512 threads cache a part of their tables and run up to 2.6 times slower)
+    int64_t base = threads <= 512 ? 192 : step_has_transcendentals() ? 88 : 104;
+    // (a per-element step body without exponentials or logarithms keeps few values alive besides the cached ones)
+    // The driver reads the spill count of the compiled code object and asks again with a smaller share when the
+    // register allocator did not get by.
+    return std::max<int64_t>(base * opts.reg_budget_scale / 100, 8);
   }
 
   // whether the per-element body of a step loop (a thread-mapped loop inside a sequential loop) takes exponentials

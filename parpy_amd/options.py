@@ -262,6 +262,9 @@ class CompileOptions:
         'opt_fence_iterations': None,
         'opt_prefetch_steps': None,
         'reg_budget': None,   # registers per thread the caching passes may claim (None: by block size)
+        'reg_budget_scale': None,   # percent of the default budget (set by the register feedback of the driver)
+        'reg_feedback': True,   # recompile with a smaller budget when the code object reports spilled vector registers
+        'reg_feedback_timed': False,   # ... and pick between the two by timing them on the first call (runs the function several times)
         'assume_aligned': None,   # set by the driver: False when an array argument is not 16-byte aligned
     }
 

@@ -803,3 +803,49 @@ def test_buffers_reject_strided_and_read_only_arrays():
         parpy.print_compiled(K.axpy, [1.0, ro, ro, ro, 8], opts_for({'N': parpy.threads(8)}))
     with pytest.raises(RuntimeError, match="nested dictionary"):
         parpy.print_compiled(K.dict_scale, [{"n": {"a": 1}}, x], opts_for({'N': parpy.threads(8)}))
+
+
+def test_code_object_metadata_and_register_feedback():
+    """The registers a compiled kernel was given are read from the metadata note of its code object; a function whose
+    code object reports spilled vector registers is compiled again with smaller budgets for the caching passes and
+    the version that spills least is the one that is kept."""
+    from parpy_amd import codeobject
+    import parpy_amd
+    hmm, seqs, args = _hmm_args(7, n=2, maxlen=12)
+    args = [W.with_scaled_tables(args[0]), args[1], np.zeros(2, dtype=np.float64)] + args[3:]
+    o = opts_for({'inst': parpy.threads(2), 'state': parpy.threads(1024)})
+    s = parpy.print_compiled(W.forward_scaled, args, o)
+    res = codeobject.kernel_resources(hiprtc_compile(s[:s.index("// host side")], o))
+    step = [v for k, v in res.items() if k.startswith("forward_scaled_inst")]
+    assert len(step) == 1 and 64 < step[0]["vgprs"] <= 128 and step[0]["lds_bytes"] >= 2 * 65536 and step[0]["max_threads"] == 1024
+    assert step[0]["spilled_vgprs"] == 0 and step[0]["scratch_bytes"] == 0      # the headline kernel at its default budget
+    # a budget far beyond the register file of a 1024-thread workgroup spills ...
+    o.reg_budget = 160
+    s = parpy.print_compiled(W.forward_scaled, args, o)
+    assert codeobject.spilled_vgprs(hiprtc_compile(s[:s.index("// host side")], o)) > 0
+    # ... and the feedback loop, started from a code object that spills, ends on one that spills less
+    calls = []
+    real = parpy_amd.compiler.compile_ir
+
+    def spy(ir_ast, a, opts, tops=None):
+        calls.append(opts.reg_budget_scale)
+        if opts.reg_budget_scale is None:      # stand in for an estimate that was too generous
+            o2 = __import__("copy").copy(opts)
+            o2.reg_budget = 160
+            return real(ir_ast, a, o2, tops)
+        return real(ir_ast, a, opts, tops)
+    import pytest as _pytest
+    mp = _pytest.MonkeyPatch()
+    try:
+        mp.setattr(parpy_amd.compiler, "compile_ir", spy)
+        import parpy_amd.compile as C
+        mp.setattr(C, "get_wrapper", lambda name, key, plan, opts: ("wrapper", key))
+        from parpy_amd.validate import check_arguments
+        o3 = opts_for({'inst': parpy.threads(2), 'state': parpy.threads(1024)}, backend=parpy.CompileBackend.Hip)
+        ir = parpy_amd._ir_asts[W.forward_scaled]
+        w = parpy_amd._compile_function(ir, check_arguments(args, o3, False), o3)
+    finally:
+        mp.undo()
+    assert calls[0] is None and 80 in calls
+    with open(C._get_code_path(w[1]), "rb") as f:
+        assert codeobject.spilled_vgprs(f.read()) == 0
