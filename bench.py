@@ -52,12 +52,15 @@ OPT_FLAGS = ("opt_vectorize", "opt_lds_rows", "opt_reg_cache", "opt_hoist_invari
 # waves per read puts S / 256 rows of 64 states on each SIMD.  The issue times of the two classes and the LDS rates
 # are measured by microkernels in the same run (`measure_rates`); the figures below are what those measured when the
 # committed profiles were taken (profiles/valu_rates.md, profiles/lds_rates.md) and serve as a cross-check only.
-COMMITTED_VALU_NS = {"full": 1.02, "trans": 3.63}
+COMMITTED_VALU_NS = {"fast": 1.02, "normal": 2.03, "trans": 3.63}
 COMMITTED_LDS_GBS_PER_CU = {"read32": 245.5, "read64": 463.0, "read128": 465.9, "write32": 147.5, "write64": 197.7, "write128": 178.9}
+# Per state and step: instructions of the double-rate class (v_add / v_sub / v_mul / v_fma_f32), of the single-rate
+# class (v_max / v_min, integer and address arithmetic, selects) and transcendentals (SQ_INSTS_VALU_* counters of the
+# 7-mer kernels, profiles/hmm7_valu_classes.md).
 HMM_VALU_MIX = {
-    "reference": {"full": 24.0, "trans": 6.0},
-    "grouped": {"full": 14.2, "trans": 3.0},
-    "scaled": {"full": 8.4, "trans": 0.0},
+    "reference": {"fast": 21.0, "normal": 3.57, "trans": 6.0},
+    "grouped": {"fast": 11.25, "normal": 2.5, "trans": 3.0},
+    "scaled": {"fast": 7.04, "normal": 1.91, "trans": 0.0},
 }
 HMM_FORMS = {"scaled": "forward_scaled", "grouped": "forward_syn4", "reference": "forward_syn"}
 # LDS bytes per state and step: the grouped and scaled forms read one predecessor word (4-byte reads, issued two to
@@ -126,15 +129,22 @@ def _hmm_bounds(form, S, longest, kernel_ms, rates):
     mix = HMM_VALU_MIX[form]
     rows_per_simd = S / 256.0
     ns = rates["valu_ns"]
-    valu_ms = longest * rows_per_simd * (mix["full"] * ns["full"] + mix["trans"] * ns["trans"]) * 1e-6
+    parts_ns = mix["fast"] * ns["fast"] + mix["normal"] * ns["normal"] + mix["trans"] * ns["trans"]
+    replay_ns = ns["replay_ns_per_state"][form]
+    valu_ms = longest * rows_per_simd * replay_ns * 1e-6
+    parts_ms = longest * rows_per_simd * parts_ns * 1e-6
     gbs = rates["lds_gbs_per_cu"]
     lds_ms = longest * S * sum(b / (gbs[kind] * 1e9) for kind, b in HMM_LDS_MIX[form].items()) * 1e3
     clk = sum(b / VENDOR_LDS_BYTES_PER_CLK["read" if kind.startswith("read") else "write"] for kind, b in HMM_LDS_MIX[form].items())
     vendor_ms = longest * S * clk / (PEAK_CLOCK_GHZ * 1e9) * 1e3
     return {
         "valu_bound": {"ms": valu_ms, "frac": valu_ms / kernel_ms, "rates": rates["source"],
-                       "model": f"{longest} steps of the longest read x {rows_per_simd:g} rows of 64 states per SIMD x "
-                                f"({mix['full']} full-rate x {ns['full']:.3g} ns + {mix['trans']} exp/log x {ns['trans']:.3g} ns)"},
+                       "model": f"{longest} steps of the longest read x {rows_per_simd:g} rows of 64 states per SIMD x {replay_ns:.3g} ns: a "
+                                f"register-only replay of the step's instruction classes per state ({mix['fast']} double-rate, "
+                                f"{mix['normal']} single-rate, {mix['trans']} exp/log), four waves per SIMD",
+                       "sum_of_parts_ms": parts_ms, "sum_of_parts_frac": parts_ms / kernel_ms,
+                       "sum_of_parts": f"{mix['fast']} x {ns['fast']:.3g} ns + {mix['normal']} x {ns['normal']:.3g} ns + {mix['trans']} x {ns['trans']:.3g} ns "
+                                       "per state (each class measured alone)"},
         "lds_bound": {"ms": lds_ms, "frac": lds_ms / kernel_ms, "rates": rates["source"],
                       "model": f"{longest} steps of the longest read x {S} states x "
                                + " + ".join(f"{b} B {kind} at {gbs[kind]:.4g} GB/s" for kind, b in HMM_LDS_MIX[form].items())
@@ -501,18 +511,27 @@ def _lds_rates(torch, parpy):
 
 
 def _valu_rates(torch, parpy):
-    """Issue time of a full-rate vector instruction and of v_exp_f32 per wave with four waves on a SIMD (a
-    1024-thread workgroup on its compute unit, 100 compute units busy): register-only microkernels."""
+    """Issue times per wave instruction with four waves on a SIMD (a 1024-thread workgroup on its compute unit, 100
+    compute units busy), register-only microkernels: the double-rate class, the single-rate class, transcendentals,
+    and -- per statement of the HMM step -- a replay of the instruction classes of 16 states in the proportions the
+    hardware counters report for the kernel (`replay_ns_per_state`): mixing transcendentals with other
+    instructions costs more than the sum of the parts, however they are ordered, and the replay includes that."""
     o = parpy.CompileOptions()
     o.backend = parpy.CompileBackend.Hip
     iters, blocks = 20000, 100
     out = torch.zeros(blocks * 1024, dtype=torch.float32, device="cuda")
-    res = {}
-    for key, name, adds, exps in (("full", "valu_add32", 32, 0), ("trans", "valu_exp8", 0, 8)):
-        f = parpy.compile_string(name, _valu_rate_kernel(name, adds, exps), o, grid=(blocks, 1, 1), block=(1024, 1, 1))
+    res = {"replay_ns_per_state": {}}
+    jobs = [("fast", "valu_add32", "a" * 32, 32), ("normal", "valu_max32", "m" * 32, 32), ("trans", "valu_exp8", "e" * 8, 8)]
+    jobs += [("replay:" + form, "valu_replay_" + form, _replay_pattern(mix), 16) for form, mix in HMM_VALU_MIX.items()]
+    for key, name, pattern, per in jobs:
+        f = parpy.compile_string(name, _valu_rate_kernel(name, pattern), o, grid=(blocks, 1, 1), block=(1024, 1, 1))
         t = _median_wall(f, (out, 10), (out, iters), parpy, torch, o.backend)
-        # four waves per SIMD take turns: the time of one instruction of one wave is the loop time over 4 x count
-        res[key] = t * 1e9 / (iters * 4 * (adds + exps))
+        # four waves per SIMD take turns: the time of one instruction (or state) of one wave is the loop time over 4 x count
+        v = t * 1e9 / (iters * 4 * per)
+        if key.startswith("replay:"):
+            res["replay_ns_per_state"][key[7:]] = v
+        else:
+            res[key] = v
     return res
 
 
@@ -562,10 +581,20 @@ def bench_lds_rates(args, torch, parpy, W, default_cfg=True):
             "roofline": None, "cpu_baseline": None}
 
 
-def _valu_rate_kernel(name, adds, exps):
-    """A loop whose body is `adds` independent v_add_f32 (eight accumulators) and `exps` independent v_exp_f32, registers only."""
-    lines = [f"v_add_f32 v{16 + i % 8}, v{16 + i % 8}, v{41 + i % 8}" for i in range(adds)]
-    lines += [f"v_exp_f32 v{24 + i % 8}, v{24 + i % 8}" for i in range(exps)]
+def _valu_rate_kernel(name, pattern):
+    """A loop whose body is the instruction string `pattern` on registers only: 'a' an independent v_add_f32 (eight
+    accumulators; the double-rate class), 'm' a v_max_f32 (the single-rate class), 'e' a v_exp_f32."""
+    lines, na, ne = [], 0, 0
+    for ch in pattern:
+        if ch == "a":
+            lines.append(f"v_add_f32 v{16 + na % 8}, v{16 + na % 8}, v{41 + na % 8}")
+            na += 1
+        elif ch == "m":
+            lines.append(f"v_max_f32 v{16 + na % 8}, v{16 + na % 8}, v{41 + na % 8}")
+            na += 1
+        else:
+            lines.append(f"v_exp_f32 v{24 + ne % 8}, v{24 + ne % 8}")
+            ne += 1
     body = "\\n".join(lines)
     init = "\\n".join([f"v_mov_b32 v{r}, 0x3f000000" for r in range(40, 52)] + [f"v_mov_b32 v{r}, 0" for r in range(16, 32)])
     clob = ", ".join(f'"v{r}"' for r in range(16, 32))
@@ -582,12 +611,25 @@ extern "C" __global__ void __launch_bounds__(1024) {name}(float* out, int iters)
 }}'''
 
 
+def _replay_pattern(mix, states=16):
+    """The instruction classes of `states` states of a step, state by state: double-rate, single-rate, transcendental."""
+    out, done = [], {"fast": 0, "normal": 0, "trans": 0}
+    for k in range(1, states + 1):
+        for cls, ch in (("fast", "a"), ("normal", "m"), ("trans", "e")):
+            n = int(round(mix[cls] * k)) - done[cls]
+            out.append(ch * n)
+            done[cls] += n
+    return "".join(out)
+
+
 def bench_valu_rates(args, torch, parpy, W, default_cfg=True):
     """Vector-ALU issue times (the times behind `valu_bound` of the HMM records)."""
     r = measure_rates(args, torch, parpy)
-    return {"metric": "vector-ALU issue time per wave instruction with 4 waves per SIMD, 1xMI355X", "value": r["valu_ns"]["full"], "unit": "ns",
+    v = r["valu_ns"]
+    return {"metric": "vector-ALU issue time per wave instruction with 4 waves per SIMD, 1xMI355X", "value": v["fast"], "unit": "ns",
             "ms_per_step": None, "higher_is_better": False, "dtype": "f32",
-            "config": {"workload": "valu_rates", "v_add_f32_ns": r["valu_ns"]["full"], "v_exp_f32_ns": r["valu_ns"]["trans"],
+            "config": {"workload": "valu_rates", "v_add_f32_ns": v["fast"], "v_max_f32_ns": v["normal"], "v_exp_f32_ns": v["trans"],
+                       "replay_ns_per_state": v["replay_ns_per_state"], "instruction_classes_per_state": HMM_VALU_MIX,
                        "shader_clock_ghz_under_valu_load": r["shader_clock_ghz_under_valu_load"]},
             "roofline": None, "cpu_baseline": None}
 
