@@ -360,11 +360,14 @@ def test_values_a_thread_stored_in_a_step_are_read_back_from_registers():
         ns = {"parpy": parpy}
         exec(compile(src, fname, "exec"), ns)
         return parpy.jit(ns[f"lookup_{first}"])
-    x = np.zeros((2, 4096), dtype=np.float32)
+    x = np.zeros((2, 8192), dtype=np.float32)
     o2 = opts_for({'i': parpy.threads(2), 'j': parpy.threads(1024)})
-    same = compiles(parpy.print_compiled(make("x", "y"), [x, x.copy(), np.zeros(2, dtype=np.float32), 2, 4096, 6], o2))
-    other = compiles(parpy.print_compiled(make("y", "x"), [x, x.copy(), np.zeros(2, dtype=np.float32), 2, 4096, 6], o2))
+    same = compiles(parpy.print_compiled(make("x", "y"), [x, x.copy(), np.zeros(2, dtype=np.float32), 2, 8192, 6], o2))
+    other = compiles(parpy.print_compiled(make("y", "x"), [x, x.copy(), np.zeros(2, dtype=np.float32), 2, 8192, 6], o2))
     assert "kept_dst" in same and "kept_" not in other
+    # (a single vector per thread is reloaded with one instruction: not kept)
+    x1 = np.zeros((2, 4096), dtype=np.float32)
+    assert "kept_" not in compiles(parpy.print_compiled(make("x", "y"), [x1, x1.copy(), np.zeros(2, dtype=np.float32), 2, 4096, 6], o2))
 
 
 def test_adjacent_accesses_are_only_packed_when_nothing_they_pass_can_touch_them():
