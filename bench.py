@@ -45,7 +45,7 @@ FP32_MATRIX_PEAK_TFLOPS = 157.3
 OPT_FLAGS = ("opt_vectorize", "opt_lds_rows", "opt_reg_cache", "opt_hoist_invariant", "opt_narrow_index", "opt_unswitch",
              "opt_gather_transpose", "opt_nontemporal", "opt_lane_split", "opt_drop_barriers", "opt_unswitch_uniform",
              "opt_offset32", "opt_if_convert", "opt_noalias_scopes", "opt_mfma_sddmm", "opt_expand_short_loops",
-             "opt_guard_bounds", "opt_prefetch_steps", "opt_pack_accesses", "opt_share_iterations", "opt_fence_iterations", "opt_keep_stored")
+             "opt_guard_bounds", "opt_prefetch_steps", "opt_pack_accesses", "opt_share_iterations", "opt_fence_iterations", "opt_keep_stored", "opt_keep_own")
 
 # Vector-ALU instructions per state and step in the time loop of the generated HMM kernels (counted in the ISA of
 # the kernels as compiled for these shapes: full-rate instructions, and v_exp_f32 / v_log_f32).  One workgroup of 16

@@ -100,7 +100,7 @@ def _compile_function(ir_ast, args, opts):
 
 def _register_feedback(ir_ast, args, opts, top_map, name, res, cache_key, path):
     """The register budgets of the caching passes are estimates; the compiled code object says how they turned
-    out.  When it reports spilled vector registers (and the budget was not set by hand) the function is
+    out.  When it reports more than four spilled vector registers (and the budget was not set by hand) the function is
     compiled again with 80 % and, if that still spills, 60 % of the budget, and the version that spills the least
     is kept.  With `opts.reg_feedback_timed` the choice is made by the clock instead: the versions for 100, 80, 60,
     45 and 30 % of the budget (those that differ) are each run and timed on the arguments of this call and the
@@ -114,7 +114,9 @@ def _register_feedback(ir_ast, args, opts, top_map, name, res, cache_key, path):
         return res, cache_key
     with open(path, "rb") as f:
         spills = spilled_vgprs(f.read())
-    if spills == 0 and not opts.reg_feedback_timed:
+    # (up to four spilled registers are left alone: each costs a scratch access per loop iteration, where the next
+    # smaller budget drops a whole cached row and pays a load per element for it)
+    if spills <= 4 and not opts.reg_feedback_timed:
         return res, cache_key
     candidates = [(spills, 100, res, cache_key)]
     seen = {res.device_src}

@@ -207,7 +207,7 @@ def describe_opts(opts):
     if opts.force_float_size is not None:
         parts.append(f"(force_float_size {opts.force_float_size.value})")
     for name in ("opt_vectorize", "opt_lds_rows", "opt_reg_cache", "opt_hoist_invariant",
-                 "opt_narrow_index", "opt_mfma_sddmm", "opt_unswitch", "opt_gather_transpose", "opt_nontemporal", "opt_lane_split", "opt_drop_barriers", "opt_unswitch_uniform", "opt_offset32", "opt_if_convert", "opt_noalias_scopes", "opt_expand_short_loops", "opt_guard_bounds", "opt_prefetch_steps", "opt_pack_accesses", "opt_share_iterations", "opt_fence_iterations", "opt_keep_stored", "assume_aligned"):
+                 "opt_narrow_index", "opt_mfma_sddmm", "opt_unswitch", "opt_gather_transpose", "opt_nontemporal", "opt_lane_split", "opt_drop_barriers", "opt_unswitch_uniform", "opt_offset32", "opt_if_convert", "opt_noalias_scopes", "opt_expand_short_loops", "opt_guard_bounds", "opt_prefetch_steps", "opt_pack_accesses", "opt_share_iterations", "opt_fence_iterations", "opt_keep_stored", "opt_keep_own", "assume_aligned"):
         v = getattr(opts, name, None)
         if v is not None:
             parts.append(f"({name} {1 if v else 0})")

@@ -388,6 +388,7 @@ struct Options {  // src/option.rs:14-108
   bool opt_prefetch_steps = true;     // loads indexed by the counter of a barrier-stepped loop are issued one step ahead
   bool opt_pack_accesses = true;      // four adjacent 4-byte accesses of one iteration become one 16-byte access
   bool opt_share_iterations = true;   // what all iterations of one thread have in common is evaluated once per thread
+  bool opt_keep_own = false;     // ... and across steps when source and destination swap every step (own elements never re-read from LDS)
   bool opt_keep_stored = true;   // values a thread stores and reads back itself later in the same step stay in registers
   bool opt_fence_iterations = true;   // the unrolled iterations of a thread that read and write LDS are scheduled one after the other
   bool opt_expand_short_loops = true; // counted loops of <= 8 iterations inside a parallel iteration are expanded in place

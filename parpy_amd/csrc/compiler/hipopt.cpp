@@ -2123,13 +2123,110 @@ struct Pass {
       r->body = keep_stored_rows(st->body, budget);
       r->els = keep_stored_rows(st->els, budget);
       bool seq = st->k == Stmt::For && st->map.k == GpuMap::None && !st->unroll;
-      if (seq) r->body = keep_in_iteration(r->body, budget);
+      if (seq) {
+        Stmts pre;
+        r->body = keep_in_iteration(r->body, budget, st, &pre);
+        for (auto& p : pre) out.push_back(p);
+      }
       out.push_back(r);
     }
     return out;
   }
 
-  Stmts keep_in_iteration(const Stmts& B, int64_t* budget) {
+  // `t & 1` on the variable of a loop with step one (possibly compared with zero): true in every other iteration
+  static bool alternates(const E& cond, const S& loop) {
+    E c = cond;
+    while (c->k == Expr::Convert) c = c->args[0];
+    if (c->k == Expr::BinOpE && c->bop == BinOp::Neq && c->args[1]->k == Expr::Int && c->args[1]->iv == 0) c = c->args[0];
+    while (c->k == Expr::Convert) c = c->args[0];
+    if (!(c->k == Expr::BinOpE && c->bop == BinOp::BitAnd && loop->step == 1)) return false;
+    E v = c->args[0], one = c->args[1];
+    while (v->k == Expr::Convert) v = v->args[0];
+    return v->k == Expr::Var && v->name == loop->id && one->k == Expr::Int && one->iv == 1;
+  }
+
+  // The second half: when the pointer pair of the step swaps its arrays every iteration (`src = a, dst = b`, the
+  // other way round when `t & 1`), what a thread reads of its own elements through `src` in one iteration is what
+  // it stored through `dst` in the iteration before.  The register array then lives across the iterations: filled
+  // from the start row in front of the loop, read where the loop read its own elements from LDS, overwritten by the
+  // stores.  A third of the LDS bytes of the rescaled HMM step (the 16-byte loads of the own states) go.
+  // Returns the rewritten body of the storing loop, or an empty list when the conditions do not hold.
+  Stmts carry_across_iterations(const Stmts& B, size_t p1, const S& L1, const IterSpace& is1, const S& seq_loop, const AliasDef& dx,
+                                int64_t V, const std::map<int64_t, size_t>& store_at, const Name& reg, ElemSize sz, Stmts* pre) {
+    Type ity = Type::scalar(isz);
+    if (!alternates(dx.cond, seq_loop) || seq_loop->lo->k != Expr::Int) return {};
+    // the pointer the own elements are read through: the swapped pair, same test
+    Name Xs;
+    bool ok = true;
+    std::map<int64_t, size_t> last_read;     // c -> last statement of the body that reads element c through Xs
+    for (size_t i = 0; i < L1->body.size() && ok; ++i)
+      visit_stmts({L1->body[i]}, [&](const S& c) {
+        visit_stmt_exprs(c, [&](const E& x) {
+          if (x->k != Expr::Index || x->args[0]->k != Expr::Var) return;
+          int64_t v = 0, k0 = 0;
+          if (!scaled_index(x->args[1], L1->id, &v, &k0) || v != V || x->ty.sz != sz) return;
+          if (c->k == Stmt::Assign && c->dst.get() == x.get()) return;      // the store itself
+          AliasDef d = alias_definition(B, p1, x->args[0]->name);
+          if (!(d.ok && d.a == dx.b && d.b == dx.a && expr_eq(d.cond, dx.cond))) return;
+          if (Xs.s.empty()) Xs = x->args[0]->name;
+          else if (!(Xs == x->args[0]->name)) ok = false;
+          last_read[k0] = i;
+        });
+      });
+    if (!ok || Xs.s.empty()) return {};
+    // an element is read before the thread overwrites it (the register slot holds the old value until then)
+    for (auto& kv : last_read)
+      if (kv.second > store_at.at(kv.first)) return {};
+    // nothing else in the iteration stores to memory through a pointer (the emission refill writes registers, the
+    // look-up only reads), so the rows change through this loop alone
+    bool clean = true;
+    for (size_t i = 0; i < B.size(); ++i) {
+      if (i == p1) continue;
+      visit_stmts({B[i]}, [&](const S& c) {
+        if (c->k == Stmt::Assign && c->dst->k == Expr::Index) clean = false;
+        if (c->k == Stmt::CallStmt || c->k == Stmt::While) clean = false;
+      });
+    }
+    if (!clean) return {};
+    auto reg_elem = [&](const E& slot) {
+      auto re = std::make_shared<Expr>();
+      re->k = Expr::RegElem;
+      re->ty = Type::scalar(sz);
+      re->name = reg;
+      re->args = {slot};
+      return E(re);
+    };
+    auto slot_of = [&](int64_t c) { return fold_expr(mk_binop(BinOp::Add, mk_binop(BinOp::Mul, is1.slot, mk_int(V, isz), ity), mk_int(c, isz), ity)); };
+    // in front of the loop: the thread's elements of the row that the first iteration reads
+    Name first = (seq_loop->lo->iv & 1) ? dx.a : dx.b;      // src is the pair swapped: b in even iterations, a in odd ones
+    Type pty = Type::pointer(sz);
+    pty.mem = Mem::LDS;
+    if (!lds_array_names().count(first)) return {};
+    Stmts fill;
+    for (int64_t c = 0; c < V; ++c) {
+      E idx = fold_expr(mk_binop(BinOp::Add, mk_binop(BinOp::Mul, mk_int(V, isz), mk_var(L1->id, ity), ity), mk_int(c, isz), ity));
+      fill.push_back(mk_assign(reg_elem(slot_of(c)), mk_index(mk_var(first, pty), idx, Type::scalar(sz))));
+    }
+    auto init = clone(L1);
+    init->body = fill;
+    init->unroll = true;
+    pre->push_back(mk_sync());       // what other threads stored into the start row is in place
+    pre->push_back(init);
+    return rewrite_stmts(L1->body, [&](const E& e) -> E {
+      if (e->k != Expr::Index || e->args[0]->k != Expr::Var || !(e->args[0]->name == Xs)) return e;
+      int64_t v = 0, k0 = 0;
+      if (!scaled_index(e->args[1], L1->id, &v, &k0) || v != V) return e;
+      return reg_elem(slot_of(k0));
+    });
+  }
+
+  std::set<Name> lds_array_names() const {
+    std::set<Name> r;
+    visit_stmts(k.body, [&](const S& c) { if (c->k == Stmt::LdsDecl) r.insert(c->id); });
+    return r;
+  }
+
+  Stmts keep_in_iteration(const Stmts& B, int64_t* budget, const S& seq_loop, Stmts* pre) {
     Type ity = Type::scalar(isz);
     for (size_t p1 = 0; p1 < B.size(); ++p1) {
       const S& L1 = B[p1];
@@ -2221,9 +2318,11 @@ struct Pass {
             re->args = {slot};
             return E(re);
           };
+          Stmts carried = opts.opt_keep_own ? carry_across_iterations(B, p1, L1, is1, seq_loop, dx, V, store_at, reg, sz, pre) : Stmts();
+          const Stmts& body1 = carried.empty() ? L1->body : carried;
           Stmts nb1;
-          for (size_t i = 0; i < L1->body.size(); ++i) {
-            const S& c = L1->body[i];
+          for (size_t i = 0; i < body1.size(); ++i) {
+            const S& c = body1[i];
             int64_t cc = -1;
             for (auto& kv : store_at) if (kv.second == i) cc = kv.first;
             if (cc < 0) { nb1.push_back(c); continue; }
@@ -2249,8 +2348,9 @@ struct Pass {
           decl->ty = Type::scalar(sz);
           decl->iv = slots;
           Stmts nb;
+          if (!carried.empty()) pre->insert(pre->begin(), S(decl));      // the array lives across the iterations
           for (size_t i = 0; i < B.size(); ++i) {
-            if (i == p1) { nb.push_back(decl); nb.push_back(n1); continue; }
+            if (i == p1) { if (carried.empty()) nb.push_back(decl); nb.push_back(n1); continue; }
             if (i == p2) {
               if (list == &B) nb.push_back(n2);
               else {

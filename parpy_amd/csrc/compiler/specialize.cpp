@@ -97,6 +97,7 @@ Options parse_options(const std::string& sexpr) {
     else if (h == "opt_share_iterations") o.opt_share_iterations = flag();
     else if (h == "opt_fence_iterations") o.opt_fence_iterations = flag();
     else if (h == "opt_keep_stored") o.opt_keep_stored = flag();
+    else if (h == "opt_keep_own") o.opt_keep_own = flag();
     else if (h == "opt_prefetch_steps") o.opt_prefetch_steps = flag();
     else if (h == "reg_budget") o.reg_budget = f->at(1)->as_int();
     else if (h == "reg_budget_scale") o.reg_budget_scale = f->at(1)->as_int();

@@ -261,6 +261,7 @@ class CompileOptions:
         'opt_share_iterations': None,
         'opt_fence_iterations': None,
         'opt_keep_stored': None,
+        'opt_keep_own': None,
         'opt_prefetch_steps': None,
         'reg_budget': None,   # registers per thread the caching passes may claim (None: by block size)
         'reg_budget_scale': None,   # percent of the default budget (set by the register feedback of the driver)

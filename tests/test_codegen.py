@@ -346,6 +346,15 @@ def test_values_a_thread_stored_in_a_step_are_read_back_from_registers():
     assert re.search(r"\*\(__attribute__\(\(address_space\(3\)\)\) parpy_vec4<float>\*\)&beta_dst_\d+\[\(4 \* q_\d+\)\] = pk_\d+;", step)
     off = compiles(parpy.print_compiled(W.forward_scaled, args, opts_for({'inst': parpy.threads(2), 'state': parpy.threads(1024)}, opt_keep_stored=False)))
     assert "kept_" not in off
+    # opt_keep_own (off by default: measured no faster) carries the array across the steps: source and destination
+    # swap with `t & 1`, so a thread's own states of this step are what it stored in the last one; the array is
+    # filled from the start row in front of the time loop and the step loads nothing of its own from LDS
+    own = compiles(parpy.print_compiled(W.forward_scaled, args, opts_for({'inst': parpy.threads(2), 'state': parpy.threads(1024)}, opt_keep_own=True)))
+    head, loop = own[:own.index("for (int t_")], own[own.index("for (int t_"):]
+    loop = loop[:loop.index("__syncthreads")]
+    assert re.search(r"float kept_beta_dst_\d+\[16\];", head) and len(re.findall(r"kept_beta_dst_\d+\[[^\]]*\] = pk_\d+\.[xyzw];", head)) == 4
+    assert not re.search(r"const parpy_vec4<float> pk_\d+ = \*\(__attribute__\(\(address_space\(3\)\)\) const parpy_vec4<float>\*\)&beta_src", loop)
+    assert len(re.findall(r"kept_beta_dst_\d+\[[^\]]*\] \* inv_hmm_pstay", loop)) == 4
     # a look-up through a pointer that selects the other array of the pair under that test reads other values:
     # nothing is kept; with the same selection as the stores it is
     def make(first, second):
