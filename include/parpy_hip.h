@@ -106,8 +106,9 @@ int64_t parpy_hip_plan_graph_replays(void* plan);
 /* Loops of launches inside one kernel (the plan's `persist` statements, emitted with the
  * persistent_loops option): the counterpart of the reference's answer to launch-bound host loops
  * (src/option.rs:60-63, src/gpu/inter_block.rs:466-563 hoists such loops to the host).  The
- * kernel separates the steps by a barrier over all workgroups, so the runtime uses it only when the
- * whole grid is resident at once (occupancy query when the plan is created) and runs the loop of
+ * kernel separates the steps by a barrier over all workgroups (or over those of one value of a grid
+ * dimension each, when the steps keep those values apart: the statement names the number of such
+ * groups, one counter each), so the runtime uses it only when the whole grid is resident at once (occupancy query when the plan is created) and runs the loop of
  * launches otherwise.  The barrier's wait is bounded (PARPY_HIP_BARRIER_POLLS polls, about two
  * seconds by default): a barrier that times out makes every workgroup leave the kernel, and the next
  * parpy_sync or parpy_hip_plan_run_timed returns non-zero with a message.  This returns the number

@@ -253,7 +253,7 @@ struct Stmt {
     Alloc,      // id = device allocation of iv elements of type ty.sz
     Free,       // free id
     Launch,     // kernel launch: fname, grid/block, args
-    PersistentLaunch,  // one launch of kernel fname that runs a whole host loop of launches (kept in body) with device-wide barriers
+    PersistentLaunch,  // one launch of kernel fname that runs a whole host loop of launches (kept in body) with barriers between workgroups (iv = counters they need)
     Scope,      // { body }; with args: the pointer variables in args do not alias each other inside
     WaveReduce, // id = wave_reduce<bop>(id)
     LdsDecl,    // __shared__ ty.sz id[iv]

@@ -1232,7 +1232,7 @@ struct PlanPrinter {
           for (auto& a : s->args) os << " " << hexpr(a);
           os << ") (body ";
           stmts(s->body);
-          os << "))";
+          os << ") " << std::max<int64_t>(s->iv, 1) << ")";
           break;
         }
         case Stmt::For:

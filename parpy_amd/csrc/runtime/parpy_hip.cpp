@@ -91,6 +91,7 @@ struct HStmt {
   int64_t nbytes = 0;
   std::vector<HStmt> body, els;   // Persist: body = the loop of launches that the kernel stands for
   bool fits = false;              // Persist: every workgroup of the launch can be resident at once (checked at creation)
+  int64_t groups = 1;            // Persist: groups of workgroups that meet among themselves at the barrier (one counter each)
 };
 
 constexpr int64_t KEEP_LIMIT = int64_t(1) << 30;         // per plan
@@ -166,10 +167,12 @@ struct Plan {
   int64_t scratch_top = 0;
   struct Carved { int slot; int64_t off; };
   std::vector<Carved> carved;
-  // Loops that run inside one kernel (persist statements): counter and status word of the device-wide
-  // barrier (32 bytes of device memory, allocated when the plan is created), whether a launch since the
-  // last check may have set the status, and how many runs used such a kernel.
+  // Loops that run inside one kernel (persist statements): status word and counters of the barrier between
+  // workgroups (device memory allocated when the plan is created: the status word in the first 128 bytes, then
+  // one counter every 128 bytes, as many as the statement with the most groups of workgroups needs), whether a
+  // launch since the last check may have set the status, and how many runs used such a kernel.
   unsigned* barrier_words = nullptr;
+  int64_t barrier_counters = 0;
   bool barrier_pending = false;
   int64_t persistent_launches = 0;
 };
@@ -182,11 +185,11 @@ int32_t check_barrier_status(Plan& p) {
   if (!p.barrier_pending || !p.barrier_words) return 0;
   p.barrier_pending = false;
   unsigned status = 0;
-  if (int32_t rc = check(hipMemcpy(&status, p.barrier_words + 4, sizeof status, hipMemcpyDeviceToHost), "reading the barrier status")) return rc;
+  if (int32_t rc = check(hipMemcpy(&status, p.barrier_words, sizeof status, hipMemcpyDeviceToHost), "reading the barrier status")) return rc;
   if (status != 0) {
     // the status word is only ever cleared here, after it has been reported: a later launch of the same plan
     // finds it set, leaves at its first barrier, and cannot hide that an earlier one was cut short
-    (void)hipMemset(p.barrier_words + 4, 0, sizeof status);
+    (void)hipMemset(p.barrier_words, 0, sizeof status);
     return fail("a barrier over all workgroups of a kernel that runs a whole loop of steps timed out: the workgroups "
                 "left the kernel early and its results are incomplete (PARPY_HIP_BARRIER_POLLS sets the limit)");
   }
@@ -281,6 +284,9 @@ struct PlanBuilder {
       if (s.args.size() + 3 != p.kparams[s.kernel].size())
         throw std::runtime_error("argument count mismatch for kernel " + p.knames[s.kernel]);
       s.body = stmts(x->at(9), 1);
+      // groups of workgroups that meet among themselves, one counter each
+      s.groups = x->size() > 10 ? x->at(10)->as_int() : 1;
+      if (s.groups < 1 || s.groups > (int64_t)s.grid[0] * s.grid[1] * s.grid[2]) throw std::runtime_error("bad number of barrier groups in launch plan");
       if (p.fns[s.kernel]) {
         int per_cu = 0, cus = 0, dev = 0;
         unsigned threads = s.block[0] * s.block[1] * s.block[2];
@@ -289,11 +295,17 @@ struct PlanBuilder {
                   hipModuleOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, p.fns[s.kernel], (int)threads, 0) == hipSuccess;
         if (!ok) (void)hipGetLastError();
         s.fits = ok && (int64_t)per_cu * cus >= (int64_t)s.grid[0] * s.grid[1] * s.grid[2];
-        if (s.fits && !p.barrier_words) {
+        if (s.fits && p.barrier_counters < s.groups) {
+          // nothing of this plan has run yet: a smaller block made for an earlier statement can go
+          if (p.barrier_words) (void)hipFree(p.barrier_words);
+          p.barrier_words = nullptr;
+          p.barrier_counters = 0;
           void* w = nullptr;
-          if (hipMalloc(&w, 8 * sizeof(unsigned)) != hipSuccess) { (void)hipGetLastError(); s.fits = false; w = nullptr; }
-          else if (hipMemset(w, 0, 8 * sizeof(unsigned)) != hipSuccess) { (void)hipGetLastError(); (void)hipFree(w); s.fits = false; w = nullptr; }
+          size_t bytes = (size_t)(s.groups + 1) * 32 * sizeof(unsigned);
+          if (hipMalloc(&w, bytes) != hipSuccess) { (void)hipGetLastError(); w = nullptr; }
+          else if (hipMemset(w, 0, bytes) != hipSuccess) { (void)hipGetLastError(); (void)hipFree(w); w = nullptr; }
           p.barrier_words = (unsigned*)w;
+          if (w) p.barrier_counters = s.groups;
         }
       }
     } else if (h == "for") {
@@ -447,7 +459,7 @@ int32_t run_stmt(Plan& p, const HStmt& s) {
       const bool persist = s.op == HStmt::Persist;
       // a loop inside one kernel needs its whole grid resident, memory for the barrier and a stream that is
       // not being captured (the barrier words are cleared with a memset); otherwise the loop of launches runs
-      if (persist && !(s.fits && p.barrier_words && !p.capturing)) return run_stmts(p, s.body);
+      if (persist && !(s.fits && p.barrier_words && p.barrier_counters >= s.groups && !p.capturing)) return run_stmts(p, s.body);
       const auto& kinds = p.kparams[s.kernel];
       Packed storage[64];
       void* ptrs[64];
@@ -474,14 +486,14 @@ int32_t run_stmt(Plan& p, const HStmt& s) {
         ptrs[k] = &storage[k];
       }
       if (persist) {
-        // the counter (first 16 bytes) starts from zero in every launch; the status word 16 bytes on stays as it is
-        // until the host has read it
-        if (int32_t rc = check(hipMemsetAsync(p.barrier_words, 0, 4 * sizeof(unsigned), p.launch_stream), "clearing the barrier counter")) return rc;
+        // the counters (from 128 bytes on) start from zero in every launch; the status word in front of them stays as it
+        // is until the host has read it
+        if (int32_t rc = check(hipMemsetAsync(p.barrier_words + 32, 0, (size_t)s.groups * 32 * sizeof(unsigned), p.launch_stream), "clearing the barrier counters")) return rc;
         // polls of the counter before a workgroup gives up: about a microsecond each, two seconds by default
         unsigned limit = 1u << 21;
         if (const char* e = getenv("PARPY_HIP_BARRIER_POLLS")) limit = (unsigned)strtoul(e, nullptr, 10);
-        storage[n].p = p.barrier_words;
-        storage[n + 1].p = p.barrier_words + 4;   // 16 bytes on: both words are 16-byte aligned like every pointer argument
+        storage[n].p = p.barrier_words + 32;
+        storage[n + 1].p = p.barrier_words;
         storage[n + 2].u32 = limit;
         for (size_t k = n; k < n + 3; ++k) ptrs[k] = &storage[k];
         p.barrier_pending = true;

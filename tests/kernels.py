@@ -308,3 +308,36 @@ def pick_by_quotients(a, idx, out, N):
     parpy.label('i')
     for i in range(N):
         out[i] = a[(i // 3) % 8] + a[(idx[i] // 3) % 8]
+
+
+@parpy.jit
+def exchange_steps(a, b, N, M, T):
+    """T steps that swap source and destination; row i reads row i + 1 of what the previous step wrote, so the
+    workgroups of different rows depend on each other."""
+    parpy.label('i')
+    for i in range(N):
+        for t in range(T):
+            src = a
+            dst = b
+            if t & 1:
+                src = b
+                dst = a
+            parpy.label('j')
+            for j in range(M):
+                dst[i, j] = src[(i + 1) % N, j] + src[i, (j + 1) % M]
+
+
+@parpy.jit
+def exchange_steps_within_rows(a, b, N, M, T):
+    """The same with every row on its own: only the workgroups of one row exchange data."""
+    parpy.label('i')
+    for i in range(N):
+        for t in range(T):
+            src = a
+            dst = b
+            if t & 1:
+                src = b
+                dst = a
+            parpy.label('j')
+            for j in range(M):
+                dst[i, j] = src[i, (j + 7) % M] + src[i, (j + M // 2) % M]

@@ -578,6 +578,32 @@ def test_persistent_loops_emit_one_kernel_for_the_host_loop_and_keep_the_loop_as
     assert "parpy_grid_fits_device" not in s0 and "_steps_" not in s0
 
 
+def _plan_of(fn, args, o):
+    import parpy_amd
+    from parpy_amd.validate import check_arguments
+    return parpy_amd.compiler.compile_ir(parpy_amd._ir_asts[fn], check_arguments(args, o, False), o).plan
+
+
+def test_persistent_loops_let_the_workgroups_of_one_read_meet_among_themselves():
+    """Every access of the step to the state vectors names the read as first index, so workgroups of different reads
+    never wait for each other: the barrier counts on a counter per read (128 bytes apart) up to the workgroups of one
+    read, and the plan says how many counters the launch needs.  A step that reads a neighbouring row of what the
+    steps write keeps the barrier over the whole grid."""
+    hmm, seqs, args = _hmm_args(5)
+    o = opts_for({'inst': parpy.threads(4), 'state': parpy.threads(2048)}, persistent_loops=True, backend=parpy.CompileBackend.Hip)
+    s = compiles(parpy.print_compiled(W.forward_syn, args, o))
+    assert re.search(r"parpy_grid_barrier\(parpy_bar_counter_\d+ \+ 32u \* blockIdx\.y, parpy_bar_status_\d+, 2u,", s)
+    assert re.search(r"\(persist \d+ 2 4 1 1024 1 1 .*\) 4\)", _plan_of(W.forward_syn, args, o))
+
+    a = np.zeros((2, 4096), dtype=np.float32)
+    o = opts_for({'i': parpy.threads(2), 'j': parpy.threads(4096).tpb(256)}, persistent_loops=True, backend=parpy.CompileBackend.Hip)
+    s = compiles(parpy.print_compiled(K.exchange_steps, [a, a.copy(), 2, 4096, 10], o))
+    assert re.search(r"parpy_grid_barrier\(parpy_bar_counter_\d+, parpy_bar_status_\d+, 32u,", s)
+    assert re.search(r"\(persist .*\) 1\)", _plan_of(K.exchange_steps, [a, a.copy(), 2, 4096, 10], o))
+    s = compiles(parpy.print_compiled(K.exchange_steps_within_rows, [a, a.copy(), 2, 4096, 10], o))
+    assert re.search(r"parpy_grid_barrier\(parpy_bar_counter_\d+ \+ 32u \* blockIdx\.y, parpy_bar_status_\d+, 16u,", s)
+
+
 def test_persistent_loops_keep_the_loop_of_launches_for_arrays_of_narrow_elements():
     """Workgroups exchange data through device-scope loads and stores, which exist for elements of four bytes and
     more: a ping-pong step over float16 or int8 vectors stays a loop of launches, the float32 one becomes one kernel."""

@@ -1184,6 +1184,36 @@ def test_persistent_step_loop_on_the_synthetic_model_and_fallback_when_the_grid_
     assert np.allclose(got, want, atol=1e-5, rtol=1e-5), np.abs(got - want).max()
 
 
+@pytest.mark.parametrize("rows_depend", [True, False])
+def test_persistent_step_loop_with_a_barrier_over_the_grid_or_one_per_row(rows_depend):
+    """Steps whose rows read each other's elements meet at a barrier over the whole grid, steps whose rows stay on
+    their own at one barrier per row (24 rows of 8 workgroups); both equal the same steps in NumPy exactly (sums of
+    small integers below 2^24)."""
+    N, M, T = 24, 2048, 20
+    rng = np.random.default_rng(5)
+    a0 = rng.integers(0, 3, size=(N, M)).astype(np.float32)
+    src, dst = a0.astype(np.float64), np.zeros((N, M))
+    for t in range(T):
+        if rows_depend:
+            dst = np.roll(src, -1, axis=0) + np.roll(src, -1, axis=1)
+        else:
+            dst = np.roll(src, -7, axis=1) + np.roll(src, -(M // 2), axis=1)
+        src, dst = dst, src
+    fn = K.exchange_steps if rows_depend else K.exchange_steps_within_rows
+    outs = []
+    for persistent in (False, True):
+        a = torch.from_numpy(a0).cuda()
+        b = torch.zeros_like(a)
+        o = opts_for({'i': parpy.threads(N), 'j': parpy.threads(M).tpb(256)}, persistent_loops=persistent)
+        fn(a, b, N, M, T, opts=o)
+        parpy.sync(HIP)
+        w = parpy._compile_function(parpy._ir_asts[fn], parpy.validate.check_arguments([a, b, N, M, T], o, True), o)
+        assert w.persistent_launches() == (1 if persistent else 0)
+        outs.append((b if T & 1 else a).cpu().numpy())
+    assert np.array_equal(outs[0], outs[1])
+    assert np.array_equal(outs[1], src.astype(np.float32))
+
+
 def test_persistent_step_loop_with_values_shared_between_a_threads_iterations():
     """One thread per k-mer of a 65536-state model (16 layers = 16 iterations per thread, 16 workgroups per read)
     with the time loop inside one kernel: what the iterations share is loaded at device scope in front of the
