@@ -761,6 +761,7 @@ int32_t parpy_hip_plan_create(void* module, const char* plan_text, void** plan) 
       g_barrier_plans.insert(p);
     }
   } catch (const std::exception& e) {
+    if (p->barrier_words) (void)hipFree(p->barrier_words);   // (a statement after a persist statement was malformed)
     delete p;
     return fail(std::string("invalid launch plan: ") + e.what());
   }
