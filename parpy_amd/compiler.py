@@ -7,11 +7,13 @@ text; errors come back as (kind, message, source span) and are re-raised as
 RuntimeError / TypeError / NameError with the offending source lines attached,
 like the reference does (src/utils/err.rs:79-87, src/utils/info.rs:90-121).
 """
+import concurrent.futures
 import ctypes
 import linecache
 import os
 import pathlib
 import subprocess
+import tempfile
 
 from . import _buildstamp, frontend
 from .options import CompileBackend, LoopPar, ElemSize
@@ -19,7 +21,9 @@ from .options import CompileBackend, LoopPar, ElemSize
 CSRC = pathlib.Path(__file__).parent / "csrc" / "compiler"
 LIB_PATH = pathlib.Path(__file__).parent / "libparpy_hipc.so"
 SOURCES = ["ast.cpp", "front.cpp", "constfold.cpp", "specialize.cpp", "lower.cpp",
-           "gpu.cpp", "hipopt.cpp", "hipprint.cpp", "capi.cpp"]
+           "gpu.cpp", "hipopt.cpp", "hipopt_util.cpp", "hipopt_control.cpp", "hipopt_prefetch.cpp", "hipopt_lds.cpp",
+           "hipopt_vector.cpp", "hipopt_regs.cpp", "hipopt_keep.cpp", "hipopt_alias.cpp", "hipopt_launch.cpp",
+           "hipopt_persist.cpp", "hipprint.cpp", "capi.cpp"]
 
 _lib = None
 
@@ -37,10 +41,20 @@ def build_library(force=False):
     srcs = [CSRC / s for s in SOURCES]
     if not force and LIB_PATH.exists() and _buildstamp.is_current(LIB_PATH, _deps(), _command()):
         return LIB_PATH
-    cmd = _command() + ["-o", str(LIB_PATH)] + [str(s) for s in srcs]
-    r = subprocess.run(cmd, capture_output=True, text=True)
-    if r.returncode != 0:
-        raise RuntimeError(f"Compilation of the ParPy compiler core failed:\n{r.stdout}\n{r.stderr}")
+    # one object per source file, compiled side by side, then one link
+    with tempfile.TemporaryDirectory(prefix="parpy_hipc_") as tmp:
+        def compile_one(src):
+            obj = os.path.join(tmp, src.stem + ".o")
+            cmd = [c for c in _command() if c != "-shared"] + ["-c", "-o", obj, str(src)]
+            return obj, subprocess.run(cmd, capture_output=True, text=True)
+        with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, os.cpu_count() or 1)) as pool:
+            done = list(pool.map(compile_one, srcs))
+        failed = [r for _, r in done if r.returncode != 0]
+        if failed:
+            raise RuntimeError("Compilation of the ParPy compiler core failed:\n" + "\n".join(r.stdout + r.stderr for r in failed))
+        r = subprocess.run(_command() + ["-o", str(LIB_PATH)] + [o for o, _ in done], capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError(f"Linking the ParPy compiler core failed:\n{r.stdout}\n{r.stderr}")
     _buildstamp.write_stamp(LIB_PATH, _deps(), _command())
     return LIB_PATH
 
