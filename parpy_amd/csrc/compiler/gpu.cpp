@@ -183,7 +183,9 @@ struct Restructure {
         LoopPar spar;
         spar.nthreads = std::min<int64_t>(nblocks, DEFAULT_TPB);
         spar.reduction = true;
-        spar.tpb = par.tpb;
+        // the partial results are reduced by one workgroup, also when there are more of them than the first stage's
+        // workgroups have threads (8192 threads in workgroups of 64: 128 partial results)
+        spar.tpb = std::max(par.tpb, spar.nthreads);
         out.push_back(mk_for(bid, mk_int(0, isz), mk_int(nblocks, isz), 1,
                              {mk_assign(lhs, mk_binop(op, lhs, tmpv, ty, s->i), s->i)}, spar, s->i));
         continue;

@@ -73,6 +73,9 @@ def test_multi_block_reductions_under_two_parallel_levels(fn):
     # within one workgroup nothing is cut
     s = compiles(parpy.print_compiled(fn, [x, out, N, M], opts_for({'N': parpy.threads(N), 'M': parpy.threads(M), 'K': parpy.threads(256)})))
     assert launch(s) == [("1", "20", "10", "256", "1", "1")]
+    # more partial results than a workgroup of the first stage has threads: one workgroup of 128 threads reduces them
+    s = compiles(parpy.print_compiled(fn, [x, out, N, M], opts_for({'N': parpy.threads(N), 'M': parpy.threads(M), 'K': parpy.threads(8192).tpb(64)})))
+    assert launch(s) == [("10", "128", "20", "64", "1", "1"), ("1", "20", "10", "128", "1", "1")]
 
 
 def test_multi_block_reduction_between_two_loops_of_one_nest():

@@ -46,6 +46,7 @@ REDUCE_CASES = [
     ("outer+inner", 100, 50, lambda N, M: {'outer': parpy.threads(N), 'inner': parpy.threads(128)}),
     ("irregular", 100, 83, lambda N, M: {'outer': parpy.threads(N), 'inner': parpy.threads(M)}),
     ("multi-block", 100, 2048, lambda N, M: {'outer': parpy.threads(N), 'inner': parpy.threads(M).tpb(512)}),
+    ("many small blocks", 7, 9000, lambda N, M: {'outer': parpy.threads(N), 'inner': parpy.threads(8192).tpb(64)}),
 ]
 
 
@@ -63,6 +64,8 @@ def test_reductions(fn, case):
         p = {'outer': p.get('inner', p['outer'])} if case[0] != "outer" else p
         if case[0] == "multi-block":
             p = {'outer': parpy.threads(2048).tpb(512)}
+        if case[0] == "many small blocks":
+            p = {'outer': parpy.threads(8192).tpb(64)}
     out = np.zeros(N, dtype=np.float32)
     parpy.jit(fn)(x, out, N, opts=opts_for(p))
     want = np_reduce(fn, x)
@@ -72,7 +75,8 @@ def test_reductions(fn, case):
 
 @pytest.mark.parametrize("fn", K.PLANE_REDUCTIONS, ids=lambda f: f.__name__)
 @pytest.mark.parametrize("inner", [("one workgroup", lambda: parpy.threads(256)), ("2 blocks", lambda: parpy.threads(2048)),
-                                   ("8 blocks of 128", lambda: parpy.threads(1024).tpb(128))], ids=lambda c: c[0])
+                                   ("8 blocks of 128", lambda: parpy.threads(1024).tpb(128)),
+                                   ("128 blocks of 64", lambda: parpy.threads(8192).tpb(64))], ids=lambda c: c[0])
 def test_reductions_under_two_parallel_levels(fn, inner):
     """sum / prod / max / min over the last axis of a 10 x 20 x 5000 array, the innermost level within one workgroup
     and across several (partial results per block in a device temporary, a second kernel reduces them)."""
