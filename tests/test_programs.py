@@ -94,6 +94,27 @@ def mul_planes(x, y, out):
 
 
 # ---------------------------------------------------------------- inputs
+def axpy(a, x, y, out, N):
+    """The statement of test/test_axpy.py:9-11: a labelled slice statement with a scalar taken from a tensor."""
+    parpy.label('i')
+    out[:] = a * x[:] + y[:]
+
+
+def collatz(out, N):
+    """The loop of test/test_collatz.py:9-20: a while loop of data-dependent length per element."""
+    parpy.label('i')
+    for i in range(1, N + 1):
+        v = i
+        count = 0
+        while v > 1:
+            if v % 2 == 0:
+                v = v / 2
+            else:
+                v = 3 * v + 1
+            count = count + 1
+        out[i] = count
+
+
 def syrk_data():
     M, N = 20, 30
     C = np.fromfunction(lambda i, j: ((i * j + 2) % N) / M, (N, N), dtype=np.float32).astype(np.float32)
@@ -155,7 +176,39 @@ def test_other_programs_compile():
                                                np.zeros((10, 15), dtype=np.float32)], opts_for({'N': parpy.threads(64), 'M': parpy.threads(64)})))
 
 
+def test_axpy_and_collatz_compile_and_need_parallelism():
+    import torch
+    N = 100
+    a = torch.randn(1, dtype=torch.float32)[0]            # a 0-d tensor, as in the reference's test
+    x, y = torch.randn(N), torch.randn(N)
+    s = compiles(parpy.print_compiled(axpy, [a, x, y, torch.zeros_like(x), N], opts_for({'i': parpy.threads(128)})))
+    assert re.search(r"<<<dim3\(1, 1, 1\), dim3\(128, 1, 1\)", s)
+    with pytest.raises(RuntimeError, match="does not contain any parallelism"):
+        parpy.print_compiled(axpy, [a, x, y, torch.zeros_like(x), N], opts_for({}))
+    s = compiles(parpy.print_compiled(collatz, [np.zeros(1001, dtype=np.int32), 1000], opts_for({'i': parpy.threads(128)})))
+    assert "while (" in s
+
+
 # ---------------------------------------------------------------- results (GPU)
+@pytest.mark.gpu
+def test_axpy_and_collatz():
+    import torch
+    torch.manual_seed(1234)
+    N = 100
+    a = torch.randn(1, dtype=torch.float32)[0]
+    x, y = torch.randn(N), torch.randn(N)
+    want = torch.zeros_like(x)
+    axpy(a, x, y, want, N)
+    got = torch.zeros_like(x)
+    parpy.jit(axpy)(a, x, y, got, N, opts=opts_for({'i': parpy.threads(128)}))
+    assert torch.allclose(want, got, atol=1e-5)
+    want = np.zeros(1001, dtype=np.int32)
+    collatz(want, 1000)
+    got = np.zeros(1001, dtype=np.int32)
+    parpy.jit(collatz)(got, 1000, opts=opts_for({'i': parpy.threads(256)}))
+    assert np.array_equal(got, want)
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("p", SYRK_PAR, ids=lambda p: "+".join(p))
 def test_syrk(p):
