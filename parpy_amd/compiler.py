@@ -215,7 +215,8 @@ def describe_opts(opts):
     parts = [f"(par {' '.join(par)})", f"(backend {backend})",
              f"(debug_print {1 if opts.debug_print else 0})",
              f"(use_graphs {1 if opts.use_cuda_graphs else 0})",
-             f"(persistent_loops {1 if getattr(opts, 'persistent_loops', False) else 0})"]
+             f"(persistent_loops {1 if getattr(opts, 'persistent_loops', False) else 0})",
+             f"(device_functions {1 if getattr(opts, 'device_functions', False) else 0})"]
     if opts.force_int_size is not None:
         parts.append(f"(force_int_size {opts.force_int_size.value})")
     if opts.force_float_size is not None:

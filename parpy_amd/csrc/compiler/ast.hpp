@@ -127,6 +127,7 @@ struct NameGen {
 // ---------------------------------------------------------------- expressions
 struct Expr;
 using E = std::shared_ptr<const Expr>;
+struct FunDef;
 
 // Signature of an externally defined device function (parpy.external): what a call site needs to
 // type its arguments and what the printer needs to emit the call and the include.
@@ -167,6 +168,9 @@ struct Expr {
   std::vector<E> dim_idx;
   std::vector<int64_t> dim_shape;
   std::shared_ptr<const ExtSig> ext;  // Call only: the external the call refers to
+  // Call only, when calls of jitted functions inside expressions are kept (device_functions option): before type
+  // checking the callee as parsed, afterwards its instance for the argument types of this call
+  std::shared_ptr<const FunDef> callee;
 };
 
 E mk_var(const Name& n, const Type& ty, const Info& i = Info());
@@ -345,6 +349,9 @@ struct FunDef {
   Stmts body;
   Type res_ty;
   Info i;
+  // functions called inside expressions that stay functions on the device (device_functions option): one typed
+  // instance per callee and argument types, callees before their callers
+  std::vector<std::shared_ptr<const FunDef>> device_funs;
 };
 
 // Function as parsed at decoration time: untyped, labels attached, callees inlined.
@@ -352,6 +359,13 @@ struct ParsedFun {
   std::shared_ptr<const ExtSig> ext;  // set for an external declaration (fun then only carries the name)
   FunDef fun;
   NameGen gen;
+  // the same function with the calls of jitted functions inside expressions kept as calls (statement calls are
+  // inlined in both): what the device_functions option compiles
+  FunDef fun_calls;
+  NameGen gen_calls;
+  // set when the function can only be compiled with its callees as functions (a callee returns from inside a loop):
+  // reported when it is compiled without the device_functions option
+  std::shared_ptr<const CompileError> inline_error;
   std::string source_text;  // printable form, used for cache keys
 };
 
@@ -363,6 +377,7 @@ struct Options {  // src/option.rs:14-108
   bool debug_print = false;
   Backend backend = Backend::Hip;
   bool use_graphs = false;
+  bool device_functions = false;  // jitted functions called inside expressions become device functions instead of being inlined
   bool persistent_loops = false;  // host loops of launches run inside one kernel, steps separated by a barrier over all workgroups
   bool has_force_int = false, has_force_float = false;
   ElemSize force_int = ElemSize::I64, force_float = ElemSize::F64;
@@ -427,6 +442,7 @@ struct Program {
   Stmts host;                        // host statements (loops, allocs, launches)
   std::vector<std::string> includes;
   std::vector<std::string> preamble; // device helper definitions needed by the kernels
+  std::vector<FunDef> device_funs;   // typed and lowered functions the kernels call, callees before their callers
 };
 
 // pretty printers (debug / cache key)

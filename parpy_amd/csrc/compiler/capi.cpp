@@ -76,7 +76,8 @@ int32_t parpy_hipc_compile(const parpy_hipc_fun* f, const char* args, const char
   return guarded([&] {
     std::vector<ArgDesc> a = parse_args(args);
     Options opts = parse_options(opts_text);
-    NameGen gen = f->pf->gen;  // the parsed function is shared: every compilation numbers its names from the same start
+    // the parsed function is shared: every compilation numbers its names from the same start
+    NameGen gen = opts.device_functions ? f->pf->gen_calls : f->pf->gen;
     std::ostringstream dbg;
     // every dump carries the time since the start of the compilation (src/utils/debug.rs:10-37)
     auto t0 = std::chrono::steady_clock::now();

@@ -331,6 +331,38 @@ Stmts associate_labels(const Stmts& ss) {
 struct Inliner {
   NameGen& gen;
   const std::map<std::string, const ParsedFun*>& tops;
+  // Calls of jitted functions inside expressions stay calls (for the device_functions option) when the callee only
+  // uses its parameters as scalars; statement calls are inlined either way.
+  bool keep_expr_calls = false;
+
+  const FunDef& body_of(const ParsedFun* pf) const {
+    if (!keep_expr_calls && pf->inline_error) throw *pf->inline_error;
+    return keep_expr_calls ? pf->fun_calls : pf->fun;
+  }
+
+  // no parameter is subscripted or sliced: the callee can take its arguments by value
+  static bool scalar_parameters_only(const FunDef& f) {
+    std::set<Name> params;
+    for (auto& q : f.params) params.insert(q.id);
+    bool ok = true;
+    std::function<void(const Stmts&)> walk = [&](const Stmts& ss) {
+      for (auto& st : ss) {
+        auto scan = [&](const E& root) {
+          visit_exprs(root, [&](const E& x) {
+            if (x->k == Expr::Slice) ok = false;
+            if (x->k == Expr::Subscript && x->args[0]->k == Expr::Var && params.count(x->args[0]->name)) ok = false;
+          });
+        };
+        scan(st->dst); scan(st->expr); scan(st->lo); scan(st->hi);
+        for (auto& a : st->args) scan(a);
+        if (!st->labels.empty() || st->k == Stmt::WithGpu || st->k == Stmt::CallStmt) ok = false;
+        walk(st->body);
+        walk(st->els);
+      }
+    };
+    walk(f.body);
+    return ok;
+  }
 
   // substitute parameters by argument expressions and give every callee-local
   // name a fresh identity in the caller
@@ -394,12 +426,17 @@ struct Inliner {
       c->ext = pf->ext;
       return c;
     }
-    const FunDef& f = pf->fun;
+    const FunDef& f = body_of(pf);
     if (f.params.size() != r->args.size())
       fail_rt(r->i, "Function " + f.id.s + " expected " + std::to_string(f.params.size()) + " arguments, but received " +
                         std::to_string(r->args.size()) + ".");
     if (f.body.empty() || !always_returns(f.body))
       fail_ty(r->i, "Unknown return type of function " + f.id.s);
+    if (keep_expr_calls && scalar_parameters_only(f)) {
+      auto c = std::make_shared<Expr>(*r);
+      c->callee = std::make_shared<FunDef>(f);
+      return c;
+    }
     Sub sub;
     for (size_t k = 0; k < f.params.size(); ++k) {
       E a = r->args[k];
@@ -515,7 +552,7 @@ struct Inliner {
       if (s->k == Stmt::CallStmt) {
         auto it = tops.find(s->fname);
         if (it == tops.end()) fail_rt(s->i, "Reference to unknown function " + s->fname + ".");
-        const FunDef& f = it->second->fun;
+        const FunDef& f = body_of(it->second);
         if (f.params.size() != s->args.size())
           fail_rt(f.i, "Function " + f.id.s + " expected " + std::to_string(f.params.size()) +
                            " arguments, but received " + std::to_string(s->args.size()) + ".");
@@ -587,9 +624,20 @@ std::unique_ptr<ParsedFun> parse_function(const std::string& sexpr,
   for (auto& s : pf->fun.body) body.push_back(sym.stmt(s));
   pf->fun.body = associate_labels(body);
 
-  Inliner inl{pf->gen, tops};
-  pf->fun.body = inl.run(pf->fun.body);
-  pf->source_text = print_fun(pf->fun);
+  pf->fun_calls = pf->fun;
+  pf->gen_calls = pf->gen;
+  Inliner keep{pf->gen_calls, tops};
+  keep.keep_expr_calls = true;
+  pf->fun_calls.body = keep.run(pf->fun_calls.body);
+  // what only the inlined form cannot express (a callee that returns from inside a loop) is reported when that form
+  // is asked for; everything else has already been reported by the run above
+  try {
+    Inliner inl{pf->gen, tops};
+    pf->fun.body = inl.run(pf->fun.body);
+  } catch (const CompileError& e) {
+    pf->inline_error = std::make_shared<CompileError>(e);
+  }
+  pf->source_text = print_fun(pf->inline_error ? pf->fun_calls : pf->fun);
   return pf;
 }
 

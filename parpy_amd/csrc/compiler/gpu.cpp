@@ -1063,6 +1063,7 @@ Program gpu_codegen(const FunDef& f, const Options& opts, NameGen& gen) {
   prog.name = f.id.s;
   prog.entry_params = f.params;
   prog.includes = opts.includes;
+  for (auto& d : f.device_funs) prog.device_funs.push_back(*d);
   Restructure rs(opts, gen);
   Stmts body = rs.run(f.body, f.params);
   HostGen hg{opts, gen, prog, {}, {}};

@@ -832,6 +832,7 @@ struct DevicePrinter {
         os << ind(n) << "}\n";
         break;
       case Stmt::Sync: os << ind(n) << "__syncthreads();\n"; break;
+      case Stmt::Return: os << ind(n) << "return " << pexpr(s->expr) << ";\n"; break;   // (device functions only)
       case Stmt::Scope:
         if (!s->args.empty()) {
           // an immediately invoked, always inlined lambda: its restrict-qualified parameters shadow
@@ -1104,6 +1105,43 @@ struct DevicePrinter {
     }
   }
 
+  // A jitted function that the kernels call (device_functions option): scalars in, a scalar out, printed through
+  // the statement printer of the kernels with the function's parameters in the place of a kernel's.
+  std::string device_function_text(const FunDef& f) {
+    Kernel k;
+    k.name = f.id.str();
+    for (auto& q : f.params) {
+      KernelParam kp;
+      kp.id = q.id;
+      kp.ty = q.ty;
+      k.params.push_back(kp);
+    }
+    k.body = f.body;
+    k.block = {1, 1, 1};
+    k.grid = {1, 1, 1};
+    k.cached_stores = true;
+    kernel = &k;
+    ranges.clear();
+    narrow_vars.clear();
+    reassigned.clear();
+    lds_decls.clear();
+    lds_arrays.clear();
+    pack_loads.clear();
+    pack_stores.clear();
+    packs.clear();
+    stream_out.clear();
+    os.str("");
+    find_reassigned(k.body, reassigned);
+    // parameters are plain local variables of the function: an assignment to one must not be mistaken for a constant
+    pstmts(k.body, 2);
+    std::ostringstream out;
+    out << "__device__ __forceinline__ " << elem_ctype(f.res_ty.sz) << " " << k.name << "(";
+    for (size_t i = 0; i < f.params.size(); ++i) out << (i ? ", " : "") << elem_ctype(f.params[i].ty.sz) << " " << f.params[i].id.str();
+    out << ") {\n" << os.str() << "}\n";
+    kernel = nullptr;
+    return out.str();
+  }
+
   std::string kernel_text(const Kernel& k) {
     kernel = &k;
     ranges.clear();
@@ -1351,6 +1389,7 @@ std::string hip_print_device(const Program& p, const Options& opts) {
   for (auto& h : headers) out << "#include " << ((h[0] == '<' || h[0] == '"') ? h : "\"" + h + "\"") << "\n";
   for (auto& d : p.preamble) out << d << "\n";
   DevicePrinter dp(opts);
+  for (auto& f : p.device_funs) out << "\n" << dp.device_function_text(f);
   for (auto& k : p.kernels) out << "\n" << dp.kernel_text(k);
   return out.str();
 }

@@ -149,6 +149,12 @@ FunDef lower(const FunDef& f, const Options& opts, NameGen& gen) {
   Lowerer lw{opts, gen};
   FunDef out = f;
   out.body = fold_stmts(lw.lower_stmts(f.body, false));
+  out.device_funs.clear();
+  for (auto& d : f.device_funs) {
+    auto c = std::make_shared<FunDef>(*d);
+    c->body = fold_stmts(lw.lower_stmts(d->body, false));
+    out.device_funs.push_back(c);
+  }
   return out;
 }
 

@@ -73,6 +73,7 @@ Options parse_options(const std::string& sexpr) {
     } else if (h == "debug_print") o.debug_print = flag();
     else if (h == "use_graphs") o.use_graphs = flag();
     else if (h == "persistent_loops") o.persistent_loops = flag();
+    else if (h == "device_functions") o.device_functions = flag();
     else if (h == "force_int_size") { o.has_force_int = parse_elem_tag(f->at(1)->atom, &o.force_int); }
     else if (h == "force_float_size") { o.has_force_float = parse_elem_tag(f->at(1)->atom, &o.force_float); }
     else if (h == "includes") { for (size_t j = 1; j < f->size(); ++j) o.includes.push_back(f->at(j)->atom); }
@@ -644,6 +645,15 @@ struct TypeChecker {
   const Options& opts;
   std::map<Name, Type> vars;
   Type res_ty = Type::vvoid();
+  // Functions called inside expressions that stay functions (device_functions option): one typed instance per callee
+  // and argument types, shared by the checker of the main function and those of the callees, callees first.
+  struct Instances {
+    std::map<std::string, std::shared_ptr<const FunDef>> by_key;
+    std::vector<std::shared_ptr<const FunDef>> in_order;
+    std::set<std::string> open;   // being checked: a function that reaches itself cannot be compiled
+    int next = 0;
+  };
+  std::shared_ptr<Instances> instances = std::make_shared<Instances>();
   std::set<Name> pending;             // result variables of inlined calls that have not been assigned yet
   std::map<Name, Type> resolved;      // ... and the type their first assignment gave them
 
@@ -806,7 +816,67 @@ struct TypeChecker {
   // and every call of one external must pass arrays of the same shapes.
   std::map<std::string, std::vector<Type>> ext_arg_types;
 
+  // A call of a jitted function that stays a call (src/py/insert_called_functions.rs:12-88 collects such callees,
+  // src/gpu/codegen.rs:573-585 makes them device functions): the callee is type-checked with the types of this call's
+  // arguments and becomes a function of its own, once per combination of argument types.
+  E fun_call(const E& e) {
+    const FunDef& f = *e->callee;
+    auto r = std::make_shared<Expr>(*e);
+    std::string key = f.id.s + "(";
+    std::vector<Type> tys;
+    for (size_t k = 0; k < e->args.size(); ++k) {
+      E a = expr(e->args[k]);
+      if (!a->ty.is_scalar())
+        fail_ty(a->i, "Found incompatible types in function call:\nargument " + std::to_string(k + 1) + " of " + f.id.s + " has type " +
+                          a->ty.str() + ", and a function called inside an expression takes scalars when it is compiled as a device function");
+      if (f.params[k].ty.k == Type::Tensor && f.params[k].ty.shape.empty()) a = ensure_scalar(a, f.params[k].ty.sz);   // annotated
+      tys.push_back(a->ty);
+      key += std::string(k ? "," : "") + elem_pyname(a->ty.sz);
+      r->args[k] = a;
+    }
+    key += ")";
+    auto it = instances->by_key.find(key);
+    if (it == instances->by_key.end()) {
+      if (instances->open.count(key)) fail_rt(e->i, "Call to unknown function " + f.id.s + " (a function cannot call itself)");
+      instances->open.insert(key);
+      TypeChecker tc(opts);
+      tc.instances = instances;
+      auto d = std::make_shared<FunDef>();
+      d->id = Name{f.id.s + "_fn" + std::to_string(++instances->next), 0};
+      d->i = f.i;
+      for (size_t k = 0; k < f.params.size(); ++k) {
+        tc.vars[f.params[k].id] = tys[k];
+        d->params.push_back(Param{f.params[k].id, tys[k], f.params[k].i});
+      }
+      Stmts body = tc.finish(tc.stmts(f.body));
+      if (!tc.res_ty.is_scalar()) fail_ty(e->i, "Unknown return type of function " + f.id.s);
+      d->res_ty = tc.res_ty;
+      // every return statement yields the common type of all of them
+      std::function<Stmts(const Stmts&)> fix = [&](const Stmts& ss) {
+        Stmts out;
+        for (auto& st : ss) {
+          auto c = std::make_shared<Stmt>(*st);
+          if (st->k == Stmt::Return) c->expr = tc.coerce(st->expr, d->res_ty);
+          c->body = fix(st->body);
+          c->els = fix(st->els);
+          out.push_back(c);
+        }
+        return out;
+      };
+      d->body = fold_stmts(fix(body));
+      instances->open.erase(key);
+      instances->by_key[key] = d;
+      instances->in_order.push_back(d);
+      it = instances->by_key.find(key);
+    }
+    r->callee = it->second;
+    r->sval = it->second->id.str();
+    r->ty = it->second->res_ty;
+    return r;
+  }
+
   E ext_call(const E& e) {
+    if (e->callee) return fun_call(e);
     if (!e->ext || e->ext->backend != (int)opts.backend) fail_rt(e->i, "Call to unknown function " + e->sval);
     const ExtSig& sig = *e->ext;
     if (sig.params.size() != e->args.size())
@@ -1026,7 +1096,8 @@ bool has_return(const Stmts& ss) {
 }  // namespace
 
 FunDef specialize(const ParsedFun& pf, const std::vector<ArgDesc>& args, const Options& opts, NameGen& gen) {
-  const FunDef& f = pf.fun;
+  if (!opts.device_functions && pf.inline_error) throw *pf.inline_error;
+  const FunDef& f = opts.device_functions ? pf.fun_calls : pf.fun;
   if (!has_parallelism(f.body, opts.parallelize))
     fail_rt(f.i, "The function " + f.id.s +
                      " does not contain any parallelism, which is not allowed. Try adding a label ('parpy.label') in "
@@ -1057,6 +1128,7 @@ FunDef specialize(const ParsedFun& pf, const std::vector<ArgDesc>& args, const O
   for (auto& p : out.params) tc.vars[p.id] = p.ty;
   body = tc.finish(tc.stmts(body));
   out.body = fold_stmts(body);
+  out.device_funs = tc.instances->in_order;
   return out;
 }
 

@@ -238,6 +238,7 @@ class CompileOptions:
         '_max_thread_blocks_per_cluster': 8,
         'use_cuda_graphs': False,
         'persistent_loops': False,   # host loops of launches run inside one kernel with device-wide barriers when the grid fits
+        'device_functions': False,   # jitted functions called inside expressions stay functions on the device instead of being inlined
         '_force_int_size': None,
         '_force_float_size': None,
         'opt_vectorize': None,

@@ -16,10 +16,12 @@ HIP = parpy.CompileBackend.Hip
 CODE_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "code")
 
 
-def opts_for(p):
+def opts_for(p, **kw):
     o = parpy.par(p)
     o.backend = HIP
     o.includes += [CODE_DIR]
+    for k, v in kw.items():
+        setattr(o, k, v)
     return o
 
 
@@ -151,7 +153,8 @@ def sum_rows_using_ext(out, x, N):
 
 
 # callees with more than one return statement (the reference keeps them as device functions,
-# src/py/insert_called_functions.rs:12-88; here they are inlined with the returned value in a variable)
+# src/py/insert_called_functions.rs:12-88; here they are inlined with the returned value in a variable unless the
+# device_functions option asks for functions)
 @parpy.jit
 def clamp_between(x, lo, hi):
     if x < lo:
@@ -192,6 +195,52 @@ def early_returns(x, y, sgn, N):
         sgn[i] = sign_of(x[i])
 
 
+# callees that only work as functions of their own: a return inside a loop, a loop of data-dependent length
+@parpy.jit
+def first_at_least(x: types.F32):
+    for k in range(4):
+        if x <= parpy.operators.float32(k):
+            return k
+    return 4
+
+
+@parpy.jit
+def halvings(n):
+    c = 0
+    while n > 1:
+        n2 = n // 2
+        c = c + 1
+        if n2 * 2 != n:
+            return -c
+        n = n2
+    return c
+
+
+@parpy.jit
+def add_any(a, b):
+    return a + b
+
+
+@parpy.jit
+def second_of(x, i):
+    return x[i + 1]
+
+
+@parpy.jit
+def function_calls(x, y, steps, idx, N):
+    parpy.label('N')
+    for i in range(N):
+        y[i] = parpy.operators.float32(first_at_least(x[i])) + add_any(x[i], y[i])
+        steps[i] = add_any(halvings(idx[i]), 1)
+
+
+@parpy.jit
+def mixed_callees(x, y, N):
+    parpy.label('N')
+    for i in range(N - 1):
+        y[i] = second_of(x, i) + add_call(x[i], 1.0)
+
+
 F = np.float32
 
 
@@ -208,19 +257,23 @@ def test_callees_with_several_returns_are_inlined_through_a_result_variable():
     x = np.zeros(10, dtype=F)
     s = compiles(parpy.print_compiled(early_returns, [x, x.copy(), np.zeros(10, dtype=np.int64), 10], opts_for({'N': parpy.threads(10)})))
     assert re.search(r"float clamp_between_result_\d+ = 0.0f;", s) and re.search(r"int64_t sign_of_result_\d+ = 0;", s)
-    with pytest.raises(RuntimeError, match="return statement inside a loop"):
-        @parpy.jit
-        def first_positive(x: types.F32):
-            for k in range(3):
-                if x > k:
-                    return k
-            return 3
+    # a callee that returns from inside a loop cannot be inlined this way: accepted when it is declared (it compiles as
+    # a device function), reported when the caller is compiled with inlined calls
+    @parpy.jit
+    def first_positive(x: types.F32):
+        for k in range(3):
+            if x > parpy.operators.float32(k):
+                return k
+        return 3
 
-        @parpy.jit
-        def use(x, y, N):
-            parpy.label('N')
-            for i in range(N):
-                y[i] = first_positive(x[i])
+    @parpy.jit
+    def use(x, y, N):
+        parpy.label('N')
+        for i in range(N):
+            y[i] = parpy.operators.float32(first_positive(x[i]))
+    with pytest.raises(RuntimeError, match="return statement inside a loop"):
+        parpy.print_compiled(use, [x, x.copy(), 10], opts_for({'N': parpy.threads(10)}))
+    compiles(parpy.print_compiled(use, [x, x.copy(), 10], opts_for({'N': parpy.threads(10)}, device_functions=True)))
     with pytest.raises(TypeError, match="Unknown return type"):
         @parpy.jit
         def maybe(x: types.F32):
@@ -232,6 +285,46 @@ def test_callees_with_several_returns_are_inlined_through_a_result_variable():
             parpy.label('N')
             for i in range(N):
                 y[i] = maybe(x[i])
+
+
+def test_expression_calls_as_device_functions():
+    """`device_functions`: what the reference does with functions called inside expressions
+    (src/py/insert_called_functions.rs:12-88, src/gpu/codegen.rs:573-585).  A callee becomes a `__device__` function
+    once per combination of argument types, callees in front of their callers; a callee that indexes a parameter is
+    inlined as before; statement calls are inlined in both modes."""
+    x = np.zeros(10, dtype=F)
+    dev = lambda p: opts_for(p, device_functions=True)
+    s = compiles(parpy.print_compiled(add_mul_nested, [x, x.copy(), 10], dev({'N': parpy.threads(10)})))
+    heads = re.findall(r"__device__ __forceinline__ float (\w+)_fn\d+\(float \w+, float \w+(?:, float \w+)?\)", s)
+    assert heads[-1] == "add_then_mul" and sorted(heads[:-1]) == ["add_call", "mul_call"], heads
+    assert re.search(r"= add_then_mul_fn\d+\(", s.split('extern "C" __global__')[1])
+    s = compiles(parpy.print_compiled(early_returns, [x, x.copy(), np.zeros(10, dtype=np.int64), 10], dev({'N': parpy.threads(10)})))
+    assert "clamp_between_result" not in s and re.search(r"__device__ __forceinline__ int64_t sign_of_fn\d+\(float", s)
+    assert len(re.findall(r"\n    return ", s[s.index("clamp_between_fn"):s.index("piecewise_fn")])) >= 2
+    # a return inside a loop, a while loop with an early return; two instances of one callee for two argument types
+    idx = np.arange(10, dtype=np.int64)
+    s = compiles(parpy.print_compiled(function_calls, [x, x.copy(), np.zeros(10, dtype=np.int64), idx, 10], dev({'N': parpy.threads(10)})))
+    assert re.search(r"float add_any_fn\d+\(float \w+, float \w+\)", s) and re.search(r"int64_t add_any_fn\d+\(int64_t \w+, int64_t \w+\)", s)
+    assert "while (" in s[s.index("halvings_fn"):s.index('extern "C" __global__')]
+    with pytest.raises(RuntimeError, match="return statement inside a loop"):
+        parpy.print_compiled(function_calls, [x, x.copy(), np.zeros(10, dtype=np.int64), idx, 10], opts_for({'N': parpy.threads(10)}))
+    # a callee that indexes its parameter is inlined, the scalar one beside it is a function
+    s = compiles(parpy.print_compiled(mixed_callees, [x, x.copy(), 10], dev({'N': parpy.threads(10)})))
+    assert "second_of" not in s and re.search(r"float add_call_fn\d+\(", s)
+    # statement calls are inlined in both modes
+    a = np.zeros((10, 15), dtype=F)
+    s = compiles(parpy.print_compiled(add_2d_inplace, [a, a.copy(), 10, 15], dev({'2d': parpy.threads(10), '1d': parpy.threads(15)})))
+    assert "__device__ __forceinline__ float add" not in s
+    # without the option nothing changes
+    s = parpy.print_compiled(add_mul_nested, [x, x.copy(), 10], opts_for({'N': parpy.threads(10)}))
+    assert "_fn1" not in s
+    with pytest.raises(TypeError, match="takes scalars"):
+        @parpy.jit
+        def whole(x, y, N):
+            parpy.label('N')
+            for i in range(N):
+                y[i] = add_any(x, y[i])
+        parpy.print_compiled(whole, [x, x.copy(), 10], dev({'N': parpy.threads(10)}))
 
 
 def test_statement_calls_with_sub_tensors():
@@ -359,6 +452,48 @@ def test_callees_with_several_returns_give_what_python_gives():
     want = np.clip(x, -1.0, 2.0) + pw
     assert np.allclose(y, want, rtol=1e-6, atol=1e-6)
     assert np.array_equal(sgn, np.sign(x).astype(np.int64))
+
+
+@pytest.mark.gpu
+def test_device_functions_give_the_results_of_the_inlined_code():
+    rng = np.random.default_rng(17)
+    dev = lambda p: opts_for(p, device_functions=True)
+    x = rng.standard_normal(10).astype(F)
+    y = np.zeros_like(x)
+    add_mul_nested(x, y, 10, opts=dev({'N': parpy.threads(10)}))
+    assert np.allclose(x ** 2, y)
+    y = np.zeros_like(x)
+    with_locals(x, y, 10, opts=dev({'N': parpy.threads(10)}))
+    assert np.allclose(y, 1.5 * x * x)
+    x = (3.0 * rng.standard_normal(500)).astype(F)
+    y0 = rng.standard_normal(500).astype(F)
+    outs = []
+    for o in (opts_for({'N': parpy.threads(500)}), dev({'N': parpy.threads(500)})):
+        y, sgn = y0.copy(), np.zeros(500, dtype=np.int64)
+        early_returns(x, y, sgn, 500, opts=o)
+        outs.append((y, sgn))
+    assert np.array_equal(outs[0][0], outs[1][0]) and np.array_equal(outs[0][1], outs[1][1])
+    # callees that exist only as functions, against the same steps in NumPy / plain Python
+    idx = rng.integers(1, 5000, 500).astype(np.int64)
+    idx[:12] = 2 ** np.arange(12)
+    y, steps = y0.copy(), np.zeros(500, dtype=np.int64)
+    function_calls(x, y, steps, idx, 500, opts=dev({'N': parpy.threads(500)}))
+    first = np.where(x <= 0, 0, np.where(x <= 1, 1, np.where(x <= 2, 2, np.where(x <= 3, 3, 4))))
+    assert np.allclose(y, first + (x + y0), rtol=1e-6, atol=1e-6)
+    def halv(n):
+        c = 0
+        while n > 1:
+            n2 = n // 2
+            c += 1
+            if n2 * 2 != n:
+                return -c
+            n = n2
+        return c
+    assert np.array_equal(steps, np.array([halv(int(n)) + 1 for n in idx]))
+    y = np.zeros(10, dtype=F)
+    xs = rng.standard_normal(10).astype(F)
+    mixed_callees(xs, y, 10, opts=dev({'N': parpy.threads(10)}))
+    assert np.allclose(y[:9], xs[1:] + (xs[:9] + 1.0))
 
 
 @pytest.mark.gpu
