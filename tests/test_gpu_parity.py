@@ -510,7 +510,8 @@ def test_forward_scaled_vs_oracle(k, threads):
 
 @pytest.mark.parametrize("flags", [{"opt_pack_accesses": False}, {"opt_prefetch_steps": False}, {"opt_expand_short_loops": False},
                                    {"opt_guard_bounds": False}, {"opt_hoist_invariant": False}, {"opt_lds_rows": False},
-                                   {"opt_keep_stored": False}, {"opt_fence_iterations": False}, {"opt_keep_own": True}],
+                                   {"opt_keep_stored": False}, {"opt_fence_iterations": False}, {"opt_keep_own": True},
+                                   {"device_functions": True}],
                          ids=lambda f: ",".join(f"{k}={int(v)}" for k, v in f.items()))
 def test_forward_scaled_each_pass_preserves_results(flags):
     hmm, seqs = W.synthetic_hmm(5, n_inst=8, min_len=50, max_len=200)
@@ -652,7 +653,8 @@ def test_forward_grouped_vs_oracle(k, threads):
 
 
 @pytest.mark.parametrize("flags", [{"opt_expand_short_loops": False}, {"opt_guard_bounds": False}, {"opt_hoist_invariant": False},
-                                   {"opt_lds_rows": False}, {"opt_if_convert": False}, {"opt_vectorize": False}],
+                                   {"opt_lds_rows": False}, {"opt_if_convert": False}, {"opt_vectorize": False},
+                                   {"device_functions": True}],
                          ids=lambda f: ",".join(f"{k}={int(v)}" for k, v in f.items()))
 def test_forward_grouped_each_pass_preserves_results(flags):
     hmm, seqs = W.synthetic_hmm(5, n_inst=8, min_len=50, max_len=200)
