@@ -316,9 +316,20 @@ struct Restructure {
     }
   }
 
+  // Only sequential for-loops are moved out of a parallel loop to make room for a synchronisation of all workgroups
+  // (src/gpu/inter_block.rs:448-633 does the same); a conditional or a while loop cannot be.
+  void refuse_grid_sync_under(const S& s) {
+    if ((s->k == Stmt::If || s->k == Stmt::While) && (contains_ib_sync(s->body) || contains_ib_sync(s->els)))
+      fail_rt(s->i, std::string("A parallel statement that spans several workgroups (more threads than fit one workgroup, or a "
+                                "reduction over them) sits under ") + (s->k == Stmt::If ? "a conditional" : "a while loop") +
+                        " inside a parallel loop, where all workgroups cannot meet; give it at most one workgroup's threads or "
+                        "move the condition into it");
+  }
+
   Stmts split_kernel(const S& loop) {
     Stmts body;
     for (auto& s : loop->body) {
+      refuse_grid_sync_under(s);
       if (s->k == Stmt::For) push_pieces(body, s, split_kernel(s));
       else if (!s->body.empty() || !s->els.empty()) {
         auto r = clone(s);

@@ -14,6 +14,9 @@ void Pass::lds_rows() {
   int64_t ext = const_extent(root);
   if (ext <= 0 || ext > root->map.n) return;  // a block must own exactly one value of the root variable
   if (k.block.y != 1 || k.block.z != 1) return;
+  // one workgroup per value of the root variable: when the loops below spread over several workgroups, each of them
+  // would copy the whole row in and out and overwrite what the others computed
+  if (k.grid.x * k.grid.y * k.grid.z != root->map.n) return;
   const Name r = root->id;
 
   std::map<Name, ArrayInfo> info;

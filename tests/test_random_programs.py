@@ -324,3 +324,137 @@ def test_walking_programs_on_device(case):
     got = np.full(4 * (N + 8), -7.0, dtype=np.float32)
     parpy.jit(f)(a.copy(), got, N, opts=opts_for({'i': parpy.threads(N)}))
     assert np.array_equal(got, want), (src, np.abs(got - want).max())
+
+
+# ---------------------------------------------------------------- stepping programs: rows that swap every step, a look-up every few steps
+def stepping_program(rng, case, period=None):
+    """A sequential loop of steps over two rows that swap roles (`src` / `dst` chosen by the step's parity), every
+    element of the new row a sum of products of elements of the old one (its own and two picked by a random index
+    pattern) times a table value selected by a per-step observation, groups of 1, 2 or 4 consecutive elements per
+    iteration; every few steps the largest element of the new row is looked up and the next step divides by it; at the
+    end the row is summed.  The shape of the rescaled forward pass, with everything that the memory passes key on
+    (group size, index patterns, look-up period, thread count) drawn at random."""
+    name = f"stepping_{case}"
+    V = int(rng.choice([1, 2, 4]))
+    P = int(rng.choice([1, 2, 3, 4, 8]))
+    if period is not None:
+        P = period
+    G = "(M // %d)" % V
+
+    def pred():
+        kind = int(rng.integers(0, 6))
+        if kind == 0:
+            return "q"
+        if kind == 1:
+            return f"({G} * {int(rng.integers(0, V))} + q)" if V > 1 else f"((q + 7) % M)"
+        if kind == 2:
+            return f"((q + {int(rng.integers(1, 9))}) % {G})"
+        if kind == 3:
+            return f"(({V} * q + {int(rng.integers(1, 5))}) % M)"
+        if kind == 4:
+            return "(q // 2)"
+        return "(M - 1 - q)"
+    lines = [f"def {name}(x, w, w2, tab, obs, a, b, out, N, M, T):", "    parpy.label('outer')", "    for i in range(N):",
+             "        parpy.label('inner')", "        for j in range(M):", "            a[i, j] = x[i, j]",
+             "        r = ops.float32(1.0)", "        for t in range(1, T):", "            src = b", "            dst = a",
+             "            if t & 1:", "                src = a", "                dst = b", "            o = obs[i, t]",
+             "            parpy.label('inner')", f"            for q in range(M // {V}):",
+             f"                p1 = src[i, {pred()}]", f"                p2 = src[i, {pred()}]"]
+    if int(rng.integers(0, 2)) or V == 1:
+        for u in range(V):
+            lines.append(f"                dst[i, {V} * q + {u}] = ((p1 * w[q, {u}] + p2 * w[q, {(u + 1) % V}] + src[i, {V} * q + {u}] * w2[{V} * q + {u}]) * r) * tab[o, {V} * q + {u}]")
+    else:
+        lines += [f"                for u in range({V}):",
+                  f"                    s = p1 * w[q, u] + p2 * w[q, ({V} - 1) - u] + src[i, {V} * q + u] * w2[{V} * q + u]",
+                  f"                    dst[i, {V} * q + u] = (s * r) * tab[o, {V} * q + u]"]
+    lines += ["            r = ops.float32(1.0)", f"            if t % {P} == 0:", "                cur = a", "                if t & 1:",
+              "                    cur = b", "                parpy.label('inner')", "                top = ops.max(cur[i, :])",
+              "                r = ops.float32(1.0) / top",
+              "        fin = a", "        if T & 1 == 0:", "            fin = b", "        parpy.label('inner')",
+              "        total = ops.sum(fin[i, :])", "        out[i] = total * r"]
+    return name, "\n".join(lines) + "\n", V
+
+
+STEPPING = list(range(10))
+
+
+def stepping_inputs(rng, N, M, T, V):
+    return (rng.uniform(0.5, 1.0, (N, M)).astype(np.float32), rng.uniform(0.1, 0.5, (M // V, V)).astype(np.float32),
+            rng.uniform(0.1, 0.5, M).astype(np.float32), rng.uniform(0.5, 1.0, (5, M)).astype(np.float32),
+            rng.integers(0, 5, (N, T)).astype(np.int8), np.zeros((N, M), dtype=np.float32), np.zeros((N, M), dtype=np.float32),
+            np.zeros(N, dtype=np.float32))
+
+
+@pytest.mark.parametrize("case", STEPPING[:4])
+def test_stepping_programs_compile(case):
+    rng = np.random.default_rng(6000 + case)
+    name, src, V = stepping_program(rng, case)
+    f = build(name, src)
+    N, M, T = 3, 256, 11
+    arrays = stepping_inputs(rng, N, M, T, V)
+    for threads in (64, 256):
+        s = parpy.print_compiled(f, list(arrays) + [N, M, T], opts_for({'outer': parpy.threads(N), 'inner': parpy.threads(threads)}))
+        hiprtc_compile(s[:s.index("// host side")], opts_for({}))
+
+
+def test_rows_shared_by_several_workgroups_stay_in_global_memory():
+    """With more threads on the inner level than one workgroup holds, a step is a launch of several workgroups per
+    row: none of them may stage the whole row in LDS and write it back (it would overwrite what the others computed).
+    With one workgroup per row the same program keeps its rows in LDS."""
+    for case in STEPPING[:3]:
+        rng = np.random.default_rng(6000 + case)
+        name, src, V = stepping_program(rng, case, period=1)
+        f = build(name, src)
+        N, M, T = 2, 2048, 9
+        arrays = stepping_inputs(rng, N, M, T, V)
+        for expand in (True, False):
+            o = opts_for({'outer': parpy.threads(N), 'inner': parpy.threads(2048)})
+            o.opt_expand_short_loops = expand
+            s = parpy.print_compiled(f, list(arrays) + [N, M, T], o)
+            assert "lds_a" not in s and "lds_b" not in s, (case, expand)
+            o = opts_for({'outer': parpy.threads(N), 'inner': parpy.threads(512)})
+            o.opt_expand_short_loops = expand
+            s = parpy.print_compiled(f, list(arrays) + [N, M, T], o)
+            assert "lds_a" in s and "lds_b" in s, (case, expand)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", STEPPING)
+def test_stepping_programs_on_device(case):
+    rng = np.random.default_rng(6000 + case)
+    name, src, V = stepping_program(rng, case)
+    f = build(name, src)
+    for N, M, T, threads in [(3, 256, 11, 64), (2, 1024, 18, 256), (2, 64, 7, 64), (1, 4096, 10, 1024)]:
+        arrays = stepping_inputs(rng, N, M, T, V)
+        want = [a.copy() for a in arrays]
+        f(*want, N, M, T)
+        got = [a.copy() for a in arrays]
+        parpy.jit(f)(*got, N, M, T, opts=opts_for({'outer': parpy.threads(N), 'inner': parpy.threads(threads)}))
+        for g, w_, label in zip(got[-3:], want[-3:], ("a", "b", "out")):
+            assert np.allclose(g, w_, rtol=2e-4, atol=1e-6), (src, N, M, T, threads, label, np.abs(g - w_).max())
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("expand", [True, False], ids=["expanded", "inner loop kept"])
+@pytest.mark.parametrize("case", STEPPING)
+def test_stepping_programs_over_several_workgroups(case, expand):
+    """2048 threads per row: every step is a launch of its own, the rows stay in global memory (a row that several
+    workgroups work on must not be staged in LDS by each of them).  A look-up that is not made in every step sits
+    under a conditional, where a reduction over several workgroups cannot be placed: refused with a message."""
+    rng = np.random.default_rng(6000 + case)
+    name, src, V = stepping_program(rng, case, period=1)
+    f = build(name, src)
+    N, M, T = 2, 2048, 9
+    arrays = stepping_inputs(rng, N, M, T, V)
+    o = opts_for({'outer': parpy.threads(N), 'inner': parpy.threads(2048)})
+    o.opt_expand_short_loops = expand
+    if case == 0:
+        _, src3, _ = stepping_program(np.random.default_rng(6000 + case), case, period=3)
+        with pytest.raises(RuntimeError, match="spans several workgroups"):
+            parpy.print_compiled(build(name + "_every_third", src3.replace(name, name + "_every_third")), list(arrays) + [N, M, T], o)
+    want = [a.copy() for a in arrays]
+    f(*want, N, M, T)
+    got = [a.copy() for a in arrays]
+    parpy.jit(f)(*got, N, M, T, opts=o)
+    for g, w_, label in zip(got[-3:], want[-3:], ("a", "b", "out")):
+        assert np.allclose(g, w_, rtol=2e-4, atol=1e-6), (src, label, np.abs(g - w_).max())
