@@ -354,6 +354,8 @@ def stepping_program(rng, case, period=None):
         if kind == 4:
             return "(q // 2)"
         return "(M - 1 - q)"
+    if case % 3 == 2:
+        return name, _max_plus_steps(name, rng, V, P, pred), V
     lines = [f"def {name}(x, w, w2, tab, obs, a, b, out, N, M, T):", "    parpy.label('outer')", "    for i in range(N):",
              "        parpy.label('inner')", "        for j in range(M):", "            a[i, j] = x[i, j]",
              "        r = ops.float32(1.0)", "        for t in range(1, T):", "            src = b", "            dst = a",
@@ -375,7 +377,26 @@ def stepping_program(rng, case, period=None):
     return name, "\n".join(lines) + "\n", V
 
 
-STEPPING = list(range(10))
+def _max_plus_steps(name, rng, V, P, pred):
+    """The same stepping structure in the (max, +) semiring: the best of three sums instead of a sum of three
+    products, the looked-up maximum subtracted instead of divided by (a Viterbi-like pass)."""
+    lines = [f"def {name}(x, w, w2, tab, obs, a, b, out, N, M, T):", "    parpy.label('outer')", "    for i in range(N):",
+             "        parpy.label('inner')", "        for j in range(M):", "            a[i, j] = x[i, j]",
+             "        r = ops.float32(0.0)", "        for t in range(1, T):", "            src = b", "            dst = a",
+             "            if t & 1:", "                src = a", "                dst = b", "            o = obs[i, t]",
+             "            parpy.label('inner')", f"            for q in range(M // {V}):",
+             f"                p1 = src[i, {pred()}]", f"                p2 = src[i, {pred()}]"]
+    for u in range(V):
+        lines.append(f"                dst[i, {V} * q + {u}] = ops.max(ops.max(p1 + w[q, {u}], p2 + w[q, {(u + 1) % V}]), src[i, {V} * q + {u}] + w2[{V} * q + {u}]) - r + tab[o, {V} * q + {u}]")
+    lines += ["            r = ops.float32(0.0)", f"            if t % {P} == 0:", "                cur = a", "                if t & 1:",
+              "                    cur = b", "                parpy.label('inner')", "                top = ops.max(cur[i, :])",
+              "                r = top",
+              "        fin = a", "        if T & 1 == 0:", "            fin = b", "        parpy.label('inner')",
+              "        total = ops.max(fin[i, :])", "        out[i] = total - r"]
+    return "\n".join(lines) + "\n"
+
+
+STEPPING = list(range(12))
 
 
 def stepping_inputs(rng, N, M, T, V):
