@@ -479,3 +479,58 @@ def test_stepping_programs_over_several_workgroups(case, expand):
     parpy.jit(f)(*got, N, M, T, opts=o)
     for g, w_, label in zip(got[-3:], want[-3:], ("a", "b", "out")):
         assert np.allclose(g, w_, rtol=2e-4, atol=1e-6), (src, label, np.abs(g - w_).max())
+
+
+# ---------------------------------------------------------------- gathers and per-thread dot products
+def gather_program(case):
+    """One thread per non-zero or per row with a sequential loop inside: sampled dot products with the second operand
+    read by columns or by rows, sums over ragged CSR rows, a maximum over a gathered row segment -- what the lane-group
+    and transposed-staging rewrites work on."""
+    name = f"gather_{case}"
+    kind = case % 4
+    if kind == 0:
+        body = ["    parpy.label('i')", "    for i in range(NNZ):", "        acc = ops.float32(0.0)", "        for k in range(K):",
+                "            acc = acc + A[rows[i], k] * B[k, cols[i]]", "        out[i] = acc * vals[i]"]
+    elif kind == 1:
+        body = ["    parpy.label('i')", "    for i in range(NNZ):", "        acc = ops.float32(0.0)", "        for k in range(K):",
+                "            acc = acc + A[rows[i], k] * BT[cols[i], k]", "        out[i] = acc + vals[i]"]
+    elif kind == 2:
+        body = ["    parpy.label('i')", "    for i in range(NR):", "        acc = ops.float32(0.0)", "        for j in range(ptr[i], ptr[i + 1]):",
+                "            acc = acc + vals2[j] * x[cidx[j]]", "        y[i] = acc"]
+    else:
+        body = ["    parpy.label('i')", "    for i in range(NNZ):", "        m = ops.float32(-ops.inf)", "        for k in range(K):",
+                "            m = ops.max(m, A[rows[i], k] - BT[cols[i], k])", "        out[i] = m"]
+    src = f"def {name}(A, B, BT, rows, cols, vals, out, ptr, cidx, vals2, x, y, NNZ, K, NR):\n" + "\n".join(body) + "\n"
+    return name, src, kind
+
+
+def gather_inputs(rng, K, NNZ, NR, NRa=64, NC=128):
+    A = rng.uniform(-1, 1, (NRa, K)).astype(np.float32)
+    B = rng.uniform(-1, 1, (K, NC)).astype(np.float32)
+    rows = np.sort(rng.integers(0, NRa, NNZ)).astype(np.int64)
+    cols = rng.integers(0, NC, NNZ).astype(np.int64)
+    lens = rng.integers(0, 40, NR)
+    ptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int64)
+    nn = max(int(ptr[-1]), 1)
+    return [A, B, np.ascontiguousarray(B.T), rows, cols, rng.uniform(-1, 1, NNZ).astype(np.float32), np.zeros(NNZ, dtype=np.float32), ptr,
+            rng.integers(0, NC, nn).astype(np.int64), rng.uniform(-1, 1, nn).astype(np.float32), rng.uniform(-1, 1, NC).astype(np.float32),
+            np.zeros(NR, dtype=np.float32)]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", range(4))
+def test_gather_programs_on_device(case):
+    name, src, kind = gather_program(case)
+    f = build(name, src)
+    rng = np.random.default_rng(7000 + case)
+    for K, NNZ, NR, tpb in [(1, 63, 1, None), (15, 1000, 50, 128), (128, 5000, 1000, None), (33, 64, 300, 64), (200, 1000, 7, None)]:
+        base = gather_inputs(rng, K, NNZ, NR)
+        want = [a.copy() for a in base]
+        f(*want, NNZ, K, NR)
+        n_it = NR if kind == 2 else NNZ
+        for lanes in (True, False):
+            got = [a.copy() for a in base]
+            o = opts_for({'i': parpy.threads(n_it) if tpb is None else parpy.threads(n_it).tpb(tpb)})
+            o.opt_lane_split = lanes
+            parpy.jit(f)(*got, NNZ, K, NR, opts=o)
+            assert np.allclose(got[6], want[6], rtol=1e-4, atol=1e-4) and np.allclose(got[11], want[11], rtol=1e-4, atol=1e-4), (src, K, NNZ, NR, tpb, lanes)
