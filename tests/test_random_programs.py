@@ -534,3 +534,78 @@ def test_gather_programs_on_device(case):
             o.opt_lane_split = lanes
             parpy.jit(f)(*got, NNZ, K, NR, opts=o)
             assert np.allclose(got[6], want[6], rtol=1e-4, atol=1e-4) and np.allclose(got[11], want[11], rtol=1e-4, atol=1e-4), (src, K, NNZ, NR, tpb, lanes)
+
+
+# ---------------------------------------------------------------- phases: consecutive parallel loops over the rows of a few arrays
+def phases_program(rng, case):
+    """Three to six consecutive parallel loops over one row each of the arrays u, v, w, every loop storing to its own
+    element of one array and reading the others at its own element or at a shifted, mirrored or halved one, the whole
+    optionally repeated by a sequential loop: what decides whether a row section may stay in a thread's registers
+    between two loops and whether the barrier between them orders anything."""
+    name = f"phases_{case}"
+    arrays = ["u", "v", "w"]
+
+    def at(arr):
+        kind = int(rng.integers(0, 7))
+        if kind <= 2:
+            return f"{arr}[i, j]"
+        if kind == 3:
+            return f"{arr}[i, (j + {int(rng.integers(1, 70))}) % M]"
+        if kind == 4:
+            return f"{arr}[i, M - 1 - j]"
+        if kind == 5:
+            return f"{arr}[i, j // 2]"
+        return f"{arr}[i, (j * 2) % M]"
+
+    def phase(indent):
+        dst = str(rng.choice(arrays))
+        others = [a for a in arrays if a != dst] + [dst]
+        a1, a2 = str(rng.choice(others)), str(rng.choice(others))
+        # the destination array is only read at the thread's own element in the loop that stores to it
+        t1 = f"{a1}[i, j]" if a1 == dst else at(a1)
+        t2 = f"{a2}[i, j]" if a2 == dst else at(a2)
+        op = str(rng.choice(["+", "-", "*"]))
+        scale = str(rng.choice(["0.5", "0.25", "1.0"]))
+        return [f"{indent}parpy.label('inner')", f"{indent}for j in range(M):", f"{indent}    {dst}[i, j] = ({t1} {op} {t2}) * {scale}"]
+    steps = int(rng.integers(0, 4))
+    lines = [f"def {name}(u, v, w, out, N, M):", "    parpy.label('outer')", "    for i in range(N):"]
+    ind = "        "
+    if steps:
+        lines.append(f"        for t in range({steps + 1}):")
+        ind = "            "
+    for _ in range(int(rng.integers(3, 7))):
+        lines += phase(ind)
+    lines += ["        parpy.label('inner')", "        s1 = ops.sum(u[i, :])", "        parpy.label('inner')", "        s2 = ops.max(w[i, :])",
+              "        out[i] = s1 + s2"]
+    return name, "\n".join(lines) + "\n"
+
+
+PHASES = list(range(16))
+
+
+@pytest.mark.parametrize("case", PHASES[:4])
+def test_phases_programs_compile(case):
+    rng = np.random.default_rng(8000 + case)
+    name, src = phases_program(rng, case)
+    f = build(name, src)
+    N, M = 3, 1000
+    arrays = [rng.uniform(-1, 1, (N, M)).astype(np.float32) for _ in range(3)] + [np.zeros(N, dtype=np.float32)]
+    for threads in (64, 256):
+        s = parpy.print_compiled(f, arrays + [N, M], opts_for({'outer': parpy.threads(N), 'inner': parpy.threads(threads)}))
+        hiprtc_compile(s[:s.index("// host side")], opts_for({}))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", PHASES)
+def test_phases_programs_on_device(case):
+    rng = np.random.default_rng(8000 + case)
+    name, src = phases_program(rng, case)
+    f = build(name, src)
+    for N, M, threads in [(3, 1000, 64), (2, 1024, 256), (5, 70, 64), (1, 4096, 1024), (2, 4096, 2048)]:
+        arrays = [rng.uniform(-1, 1, (N, M)).astype(np.float32) for _ in range(3)] + [np.zeros(N, dtype=np.float32)]
+        want = [a.copy() for a in arrays]
+        f(*want, N, M)
+        got = [a.copy() for a in arrays]
+        parpy.jit(f)(*got, N, M, opts=opts_for({'outer': parpy.threads(N), 'inner': parpy.threads(threads)}))
+        for g, w_, label in zip(got, want, "uvwo"):
+            assert np.allclose(g, w_, rtol=1e-4, atol=1e-5), (src, N, M, threads, label, np.abs(g - w_).max())
