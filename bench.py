@@ -1,7 +1,7 @@
 """Benchmark of the compiled hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
-                    [--workload all|hmm7|hmm5|hmm5ref|hmm7ref|rowsum|softmax|sddmm|sddmm_bt|copy|ldsrates|valurates] [--form scaled|grouped|reference]
+                    [--workload all|hmm7|hmm5|hmm5ref|hmm7ref|rowsum|softmax|sddmm|sddmm_bt|copy|ldsrates|valurates|stepmodes] [--form scaled|grouped|reference]
 
 A step is one pass of the compiled function over one batch of seeded synthetic
 input that is already resident in HBM.  The default run (`all`) first measures
@@ -812,6 +812,54 @@ def bench_copy(args, torch, parpy, W, default_cfg=True):
             "cpu_baseline": None}
 
 
+def bench_step_modes(args, torch, parpy, W, default_cfg=True):
+    """A host-hoisted time loop three ways -- a launch per step, the launches of a run replayed from a HIP graph, the
+    whole loop inside one kernel with a barrier per read -- on the synthetic 7-mer with 16 workgroups per read and on
+    a model of the reference's 7-mer size with 64 per read, for 1, 4, 8 and 32 reads of 300 steps.  Microseconds per
+    step (best of three timed calls); the three modes must give bit-equal results."""
+    import numpy as np
+    L = 300
+    table = {}
+
+    def run(fn, hmm, seqs, threads, reference_order, **kw):
+        hd, sd = W.to_device(hmm), W.to_device(seqs)
+        n, S = seqs["num_instances"], hmm["num_states"]
+        a1 = torch.zeros((n, S), dtype=torch.float32, device="cuda")
+        a2 = torch.zeros_like(a1)
+        res = torch.zeros(n, dtype=torch.float32, device="cuda")
+        o = parpy.par({"inst": parpy.threads(n), "state": parpy.threads(threads)})
+        for k_, v in kw.items():
+            setattr(o, k_, v)
+        fargs = [hd, sd, a1, a2, res] if reference_order else [hd, sd, res, a1, a2]
+        for _ in range(3):
+            fn(*fargs, opts=o)
+        parpy.sync(parpy.CompileBackend.Hip)
+        t = min(parpy.time_call(fn, *fargs, opts=o) for _ in range(3))
+        return res.cpu().numpy(), t * 1e3 / (L - 1)
+
+    cases = [("synthetic_7mer_16_workgroups_per_read", W.forward_syn, False, lambda n: W.synthetic_hmm(7, n_inst=n, min_len=L, max_len=L), 16384),
+             ("reference_format_7mer_64_workgroups_per_read", W.forward_kernel, True,
+              lambda n: W.random_reference_model(7, n_reads=n, min_len=L, max_len=L), 65536)]
+    for label, fn, ref_order, make, threads in cases:
+        table[label] = {}
+        for n in (1, 4, 8, 32):
+            hmm, seqs = make(n)
+            base, row = None, {}
+            for mode, kw in (("launches", {}), ("graph", {"use_cuda_graphs": True}), ("one_kernel", {"persistent_loops": True})):
+                got, us = run(fn, hmm, seqs, threads, ref_order, **kw)
+                base = got if base is None else base
+                assert np.array_equal(got, base), (label, n, mode)
+                row[mode] = round(us, 2)
+            table[label][f"reads_{n}"] = row
+    first = table["synthetic_7mer_16_workgroups_per_read"]["reads_8"]
+    return {"metric": "host-hoisted time loop: microseconds per step as launches, graph replay, one kernel", "value": first["one_kernel"],
+            "unit": "us/step", "ms_per_step": first["one_kernel"] * 1e-3, "higher_is_better": False, "dtype": "f32",
+            "config": {"workload": "step_modes", "steps_per_run": L - 1, "us_per_step": table},
+            "roofline": {"bound": "hbm", "achieved": None, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": None, "traffic": None,
+                         "note": "a comparison of launch mechanisms, not a bandwidth measurement"},
+            "cpu_baseline": None}
+
+
 def _profiled_field(name, field):
     """A figure from the committed rocprofv3 counter summary of this kernel (profiles/<name>_kernel.md), or None."""
     import re
@@ -844,7 +892,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="all", choices=["all", "hmm7", "hmm5", "hmm5ref", "hmm7ref", "rowsum", "softmax", "sddmm", "sddmm_bt", "copy", "ldsrates", "valurates"])
+    ap.add_argument("--workload", default="all", choices=["all", "hmm7", "hmm5", "hmm5ref", "hmm7ref", "rowsum", "softmax", "sddmm", "sddmm_bt", "copy", "ldsrates", "valurates", "stepmodes"])
     ap.add_argument("--form", default="scaled", choices=["scaled", "grouped", "reference"],
                     help="which statement of the HMM step is the record's value (the others are timed beside it)")
     ap.add_argument("--single-form", action="store_true", help="time only the chosen form of the HMM step (profiling runs)")
@@ -883,6 +931,7 @@ def main():
         "copy": lambda: bench_copy(args, torch, parpy, W, default_cfg),
         "ldsrates": lambda: bench_lds_rates(args, torch, parpy, W, default_cfg),
         "valurates": lambda: bench_valu_rates(args, torch, parpy, W, default_cfg),
+        "stepmodes": lambda: bench_step_modes(args, torch, parpy, W, default_cfg),
     }
     common = {"n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "scaling": "weak", "vs_baseline": None}
     runners["sddmm_bt"] = lambda: bench_sddmm(args, torch, parpy, W, default_cfg, transposed_operand=True)
