@@ -609,3 +609,114 @@ def test_phases_programs_on_device(case):
         parpy.jit(f)(*got, N, M, opts=opts_for({'outer': parpy.threads(N), 'inner': parpy.threads(threads)}))
         for g, w_, label in zip(got, want, "uvwo"):
             assert np.allclose(g, w_, rtol=1e-4, atol=1e-5), (src, N, M, threads, label, np.abs(g - w_).max())
+
+
+# ---------------------------------------------------------------- slice statements
+SLICE_SHAPES = {"x4": (5, 6, 7, 8), "x3": (6, 7, 8), "y3": (9, 8, 7), "x2": (7, 8), "y2": (8, 7), "x1": (8,), "y1": (70,), "o3": (6, 7, 8), "o2": (7, 8), "o1": (8,), "p1": (70,), "s0": (4,)}
+SLICE_INPUTS = ["x4", "x3", "y3", "x2", "y2", "x1", "y1"]
+SLICE_OUTPUTS = ["o3", "o2", "o1", "p1"]
+def slice_operand(prng, arr, extents, in_loop):
+    """A subscript of `arr` whose slice dimensions have the given extents, in order; None when it does not fit."""
+    shape = SLICE_SHAPES[arr]
+    n = len(extents)
+    if len(shape) < n: return None
+    pos = sorted(prng.choice(len(shape), size=n, replace=False).tolist())
+    parts = []
+    k = 0
+    for d, ext in enumerate(shape):
+        if k < n and d == pos[k]:
+            e = extents[k]; k += 1
+            if e > ext: return None
+            lo = int(prng.integers(0, ext - e + 1))
+            if e == ext and prng.random() < 0.6: parts.append(":")
+            elif lo == 0 and prng.random() < 0.5: parts.append(f":{e}")
+            elif lo + e == ext and prng.random() < 0.5: parts.append(f"{lo}:")
+            else: parts.append(f"{lo}:{lo + e}")
+        else:
+            if in_loop and ext >= 4 and prng.random() < 0.4: parts.append(f"i % {ext}")
+            else: parts.append(str(int(prng.integers(0, ext))))
+    return f"{arr}[{', '.join(parts)}]"
+def slice_program(prng, case):
+    name = f"slices_{case}"
+    lines = [f"def {name}(x4, x3, y3, x2, y2, x1, y1, o3, o2, o1, p1, s0):"]
+    nstmts = int(prng.integers(1, 4))
+    labels = []
+    groups = []
+    in_loop = prng.random() < 0.4
+    ind = "    "
+    if in_loop:
+        lines += ["    parpy.label('outer')", "    for i in range(4):"]
+        ind = "        "
+        labels.append("outer")
+    for sidx in range(nstmts):
+        n = int(prng.integers(1, 4))
+        extents = [int(prng.choice([1, 3, 5, 6, 7, 8])) for _ in range(n)]
+        kind = int(prng.integers(0, 3))     # 0 element-wise, 1 full reduction, 2 reduction along an axis
+        ops_in = []
+        for _ in range(int(prng.integers(1, 4))):
+            for _try in range(20):
+                o = slice_operand(prng, str(prng.choice(SLICE_INPUTS)), extents, in_loop)
+                if o: ops_in.append(o); break
+        if not ops_in: continue
+        expr = ops_in[0]
+        for o in ops_in[1:]:
+            expr = f"({expr} {str(prng.choice(['+', '-', '*']))} {o})"
+        if prng.random() < 0.3: expr = f"({expr} * 0.5)"
+        lab = [f"L{sidx}_{d}" for d in range(n)]
+        stmt = None
+        if kind == 0:
+            for _try in range(30):
+                dst = slice_operand(prng, str(prng.choice(SLICE_OUTPUTS)), extents, False)
+                if dst: stmt = f"{dst} = {expr}"; break
+        elif kind == 1:
+            red = str(prng.choice(["sum", "max", "min"]))
+            lab = lab[:int(prng.integers(0, 2))]          # a full reduction takes at most one label
+            stmt = f"s0[{int(prng.integers(0, 4))}] = ops.{red}({expr})"
+        elif n >= 2:
+            ax = int(prng.integers(0, n))
+            rest = [e for d, e in enumerate(extents) if d != ax]
+            red = str(prng.choice(["sum", "max", "min"]))
+            for _try in range(30):
+                dst = slice_operand(prng, str(prng.choice(SLICE_OUTPUTS)), rest, False)
+                if dst: stmt = f"{dst} = ops.{red}({expr}, axis={ax})"; break
+        if stmt is None: continue
+        for l in lab: lines.append(f"{ind}parpy.label('{l}')")
+        lines.append(f"{ind}{stmt}")
+        groups.append(lab)
+    if not groups: lines.append(f"{ind}parpy.label('Z')\n{ind}o1[:] = x1[:]"); groups.append(["Z"])
+    return name, "\n".join(lines) + "\n", (in_loop, groups)
+
+
+SLICES = list(range(24))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", SLICES)
+def test_slice_programs_on_device(case):
+    """One to three slice statements over arrays of one to four dimensions: element-wise assignments, full reductions
+    and reductions along an axis, with integer indices (some of them the counter of an enclosing sequential loop),
+    bounded and full slices, a label per slice dimension of which a random subset is parallel."""
+    prng = np.random.default_rng(9000 + case)
+    name, src, (in_loop, groups) = slice_program(prng, case)
+    f = build(name, src)
+    base = ([prng.uniform(-1, 1, SLICE_SHAPES[a]).astype(np.float32) for a in SLICE_INPUTS] +
+            [np.zeros(SLICE_SHAPES[a], dtype=np.float32) for a in SLICE_OUTPUTS] + [np.zeros(4, dtype=np.float32)])
+    want = [a.copy() for a in base]
+    f(*want)
+    for pick in (0, 1, 2):
+        par = {}
+        for g in groups:
+            chosen = g if pick == 0 else g[:1] if pick == 1 else g[-1:]
+            for l in chosen:
+                par[l] = parpy.threads(int(prng.choice([4, 8, 64, 128])))
+        if not par:
+            continue
+        got = [a.copy() for a in base]
+        try:
+            parpy.jit(f)(*got, opts=opts_for(par))
+        except RuntimeError as e:
+            # different thread counts on statements that end up in one kernel are refused, as in the reference
+            assert "inconsistent parallel structure" in str(e), (src, e)
+            continue
+        for g_, w_, label in zip(got[7:], want[7:], SLICE_OUTPUTS + ["s0"]):
+            assert np.allclose(g_, w_, rtol=1e-4, atol=1e-4), (src, sorted(par), label, np.abs(g_ - w_).max())
