@@ -612,9 +612,14 @@ def test_register_budgets_found_by_timing_are_within_a_tenth_of_the_best_fixed_b
                 fn(hd, sd, out, a1, a2, opts=o)
                 parpy.sync(HIP)
                 return min(parpy.time_call(fn, hd, sd, out, a1, a2, opts=o) for _ in range(3)), out.cpu().numpy().copy()
-            fixed = min(run(reg_budget=b)[0] for b in (40, 56, 72, 88, 104, 128, 160, 192, 224))
+            budgets = (40, 56, 72, 88, 104, 128, 160, 192, 224)
+            fixed = min(run(reg_budget=b)[0] for b in budgets)
             t_default, r_default = run()
             t_tuned, r_tuned = run(reg_feedback_timed=True)
+            if t_tuned > 1.1 * fixed:
+                # a sub-millisecond kernel timed once more on both sides before it counts (other work on the machine)
+                t_tuned = min(t_tuned, run(reg_feedback_timed=True)[0])
+                fixed = min(fixed, min(run(reg_budget=b)[0] for b in budgets))
             assert np.array_equal(r_default, r_tuned) or np.allclose(r_default, r_tuned, rtol=1e-6, atol=1e-3), (k, form, t_eff)
             worst.append((t_tuned / fixed, t_default / fixed, k, form, t_eff))
             # (5 % on top of the tenth for the run-to-run spread of sub-millisecond kernels)
