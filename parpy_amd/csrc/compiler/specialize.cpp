@@ -822,7 +822,9 @@ struct TypeChecker {
   E fun_call(const E& e) {
     const FunDef& f = *e->callee;
     auto r = std::make_shared<Expr>(*e);
-    std::string key = f.id.s + "(";
+    // (the text of the callee is part of the key: two functions of one name -- a callee redefined after another of
+    // its callers was declared -- are different functions)
+    std::string key = f.id.s + "#" + std::to_string(std::hash<std::string>{}(print_fun(f))) + "(";
     std::vector<Type> tys;
     for (size_t k = 0; k < e->args.size(); ++k) {
       E a = expr(e->args[k]);

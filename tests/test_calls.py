@@ -512,3 +512,29 @@ def test_externals_run():
     xf, of = rng.standard_normal((10, 64)).astype(F), np.zeros(10, dtype=F)
     sum_rows_using_ext(of, xf, 10, opts=opts_for({'N': parpy.threads(10)}))
     assert np.allclose(of, xf.sum(axis=1), atol=1e-5)
+
+
+def test_device_functions_of_one_name_with_different_bodies_stay_apart():
+    """A callee redefined after one of its callers was declared: the earlier caller keeps the earlier body, and both
+    bodies become functions of their own."""
+    @parpy.jit
+    def twice(x: types.F32):
+        return x + x
+
+    @parpy.jit
+    def uses_first(x: types.F32):
+        return twice(x) + 1.0
+
+    @parpy.jit
+    def twice(x: types.F32):      # noqa: F811  (the redefinition is the point)
+        return x * 3.0
+
+    @parpy.jit
+    def both(x, y, N):
+        parpy.label('N')
+        for i in range(N):
+            y[i] = uses_first(x[i]) + twice(x[i])
+    x = np.zeros(10, dtype=F)
+    s = compiles(parpy.print_compiled(both, [x, x.copy(), 10], opts_for({'N': parpy.threads(10)}, device_functions=True)))
+    bodies = re.findall(r"(?:float|double) twice_fn\d+\(float (\w+)\) \{\n\s+return \((.*?)\);", s)
+    assert len(bodies) == 2 and any("+" in b[1] for b in bodies) and any("* 3.0" in b[1] for b in bodies), s[s.index("__device__ __forceinline__ float twice"):][:600]
